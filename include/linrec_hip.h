@@ -202,6 +202,18 @@ size_t linrec_workspace_bytes(int64_t numseq, int64_t seqlen, int64_t row_stride
  */
 int linrec_set_spin_limit(int polls);
 
+/*
+ * The launch planner sizes grids by the number of compute units of the current device, asked once per
+ * device (hipDeviceAttributeMultiprocessorCount; the reference asks on every launch,
+ * linrec/impl/cuda/cuhelpers.cuh:23-34, linrec_pipe.cu:72-80), and by how many workgroups of the chosen
+ * kernel a CU holds.  Without a device (a plan asked for on a host without a GPU) it assumes the full
+ * part's 256.  linrec_compute_units returns the number in use.  linrec_set_compute_units overrides it
+ * for the process (tests, planning for another part); 0 returns to asking the device; the previous
+ * override is returned, and a negative argument only queries it.
+ */
+int linrec_compute_units(void);
+int linrec_set_compute_units(int cus);
+
 /* Size that serves every call with at most `max_tiles` tiles in one launch. */
 size_t linrec_workspace_bytes_for_tiles(int64_t max_tiles);
 

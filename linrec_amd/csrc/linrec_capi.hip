@@ -3,9 +3,12 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "../../include/linrec_hip.h"
 #include "colblock_kernel.hpp"
@@ -201,6 +204,65 @@ int find_kernel(int dtype, int family, int waves, int slots, int vec, int mode, 
   return -1;
 }
 
+// ---- the device ------------------------------------------------------------------------------
+// What the planner needs to know about the device a call runs on, asked once per device (the
+// reference asks through cudaDeviceGetAttribute, linrec/impl/cuda/cuhelpers.cuh:23-34, on every
+// launch, linrec_pipe.cu:72-80): the number of compute units and how many workgroups of a kernel one CU
+// holds.
+constexpr int kDefaultComputeUnits = 256;  // MI355X; assumed when a plan is asked for on a host without a GPU
+constexpr int kMaxDevices = 64;
+
+struct DeviceState {
+  std::once_flag once;
+  int cus = 0;                  // hipDeviceAttributeMultiprocessorCount
+  std::mutex occupancy_mutex;
+  std::vector<int8_t> occupancy;  // per kernel id: workgroups one CU holds, 0 = not asked yet
+};
+DeviceState g_devices[kMaxDevices];
+std::atomic<int> g_cu_override{0};
+
+// The state of the current device, set up by the first call made with that device current; nullptr if
+// there is no device to ask.
+DeviceState* device_state() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  DeviceState& d = g_devices[dev];
+  std::call_once(d.once, [&] {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) d.cus = n;
+    else (void)hipGetLastError();
+  });
+  return &d;
+}
+
+// Workgroups of kernel `id`, `block` lanes each, that one CU holds at a time; `assumed` when there is no
+// device to ask (or a test has overridden the CU count).
+int workgroups_per_cu(int id, int block, int assumed) {
+  DeviceState* d = g_cu_override.load(std::memory_order_relaxed) > 0 ? nullptr : device_state();
+  if (!d || d->cus <= 0) return assumed;
+  std::lock_guard<std::mutex> lock(d->occupancy_mutex);
+  if (d->occupancy.empty()) d->occupancy.assign(size_t(kNumKernels), 0);
+  if (d->occupancy[id] == 0) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kKernels[id].fn, block, 0) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = -1;
+    }
+    d->occupancy[id] = int8_t(std::min(n, 127));
+  }
+  return d->occupancy[id] > 0 ? d->occupancy[id] : assumed;
+}
+
+int compute_units() {
+  const int forced = g_cu_override.load(std::memory_order_relaxed);
+  if (forced > 0) return forced;
+  const DeviceState* d = device_state();
+  return d && d->cus > 0 ? d->cus : kDefaultComputeUnits;
+}
+
 // ---- planning -------------------------------------------------------------------------------
 struct Problem {
   int64_t numseq, seqlen, row_stride, elem_stride;
@@ -212,6 +274,11 @@ struct Problem {
   // batches of matrices whose rows do not continue from one matrix into the next: row r starts at
   // (r / rows_per_batch) * batch_stride + (r % rows_per_batch) * row_stride; 0 = one matrix
   int64_t rows_per_batch = 0, batch_stride = 0;
+  // Compute units of the device the call runs on.  Every row-count threshold below was measured on the
+  // full part (256 CUs) and is kept as that number; at() scales it to the device in hand, since what a
+  // threshold stands for is a number of workgroups or waves per CU.
+  int64_t cus = 256;
+  int64_t at(int64_t measured_on_256) const { return measured_on_256 * cus / 256; }
   bool batched() const { return rows_per_batch > 0 && rows_per_batch < numseq; }
 };
 
@@ -225,7 +292,7 @@ constexpr int64_t kEnoughWorkgroups = 1024;
 // Stream kernels take over from tiles for rows of more than 2048 slots once there are enough rows
 // to give every CU work.
 constexpr int64_t kLongRowSlots = 2048;  // 8192 floats, 16384 halves
-constexpr int64_t kStreamMinRows = 129;
+constexpr int64_t kStreamMinRows = 129;   // (these three on 256 CUs; scaled by Problem::at)
 constexpr int64_t kSplitBelowRows = 192;  // rows of a few thousand elements are cut into look-back tiles below this
 constexpr int64_t kSweepBelowRows = 192;  // sweep kernels take 16 .. 191 rows, stream kernels 192 .. 256
 // Fewer long rows: teams of workgroups per row, sized so that at most one workgroup per CU runs
@@ -238,12 +305,12 @@ constexpr int64_t kSweepBelowRows = 192;  // sweep kernels take 16 .. 191 rows, 
 // 35.7 / 55.3 us).
 // Sweep kernels: workgroups of a launch, two per CU forward; the backward kernels hold more
 // registers and fit one per CU.
-constexpr int64_t kSweepWorkgroupsFwd = 512;
-constexpr int64_t kSweepWorkgroupsBwd = 256;
+int64_t sweep_workgroups(const Problem& q) { return q.is_bwd ? q.cus : 2 * q.cus; }
 constexpr int64_t kSweepMaxTeam = 16;
 constexpr int64_t kSweepMinTiles = 4;  // tiles per row below which the exchange costs more than it brings
 
-constexpr int64_t kTeamWorkgroups = 256;
+// Team kernels: one workgroup per CU.
+int64_t team_workgroups(const Problem& q) { return q.cus; }
 
 // Largest divisor of `tiles_per_row` that is at most kSweepMaxTeam.
 int64_t sweep_team_size(int64_t tiles_per_row) {
@@ -275,7 +342,7 @@ int sweep_slots_for(const Problem& q, int fv) {
     // tiles of 16384 elements: the backward pass over fewer rows than the stream kernel takes (fewer
     // exchanges per byte; 16 x 1048576 backward 61.9 against 66.7 us, 64 x 524288 119 against 132 us,
     // 128 x 262144 121 against 135 us; forward the same or worse, and worse from 512 rows on)
-    if (s == 8 && !(q.is_bwd && q.numseq < kSweepBelowRows && q.seqlen / 16384 >= kSweepMinTiles &&
+    if (s == 8 && !(q.is_bwd && q.numseq < q.at(kSweepBelowRows) && q.seqlen / 16384 >= kSweepMinTiles &&
                     sweep_team_size(q.seqlen / 16384) >= kSweepMinTiles))
       continue;
     if (q.seqlen % (int64_t(8) * s * 64 * fv) == 0) { slots = s; break; }
@@ -289,14 +356,13 @@ int sweep_slots_for(const Problem& q, int fv) {
   // pass is left to one team per row where teams of 256 / rows workgroups fill the chip (bf16, 2^25
   // elements: 32 rows 72 against 83 us, 48 rows 60 against 66 us, 128 rows 72 against 86 us; 96 rows,
   // teams of 2 on 192 CUs, the same; 160 rows 62 against 50 us).
-  if (half && q.is_bwd && q.numseq <= 128 && (kTeamWorkgroups / q.numseq) * q.numseq >= 240) return 0;
-  if (q.numseq >= (half ? 32 : 16) && q.numseq < kSweepBelowRows) return slots;
+  if (half && q.is_bwd && q.numseq <= q.cus / 2 && (team_workgroups(q) / q.numseq) * q.numseq >= q.at(240)) return 0;
+  if (q.numseq >= (half ? 32 : 16) && q.numseq < q.at(kSweepBelowRows)) return slots;
   if (half) return 0;
-  if (q.numseq > 256 && (q.numseq % 256 != 0 || (q.is_bwd && (tiles_per_row < 16 || q.numseq <= 1024)))) return slots;
+  if (q.numseq > q.cus && (q.numseq % q.cus != 0 || (q.is_bwd && (tiles_per_row < 16 || q.numseq <= 4 * q.cus)))) return slots;
   return 0;
 }
-constexpr int64_t kComputeUnits = 256;
-constexpr int64_t kTailMaxRows = 96;  // rows beyond one per CU that a second launch takes
+constexpr int64_t kTailMaxRows = 96;  // rows beyond one per CU that a second launch takes (on 256 CUs)
 constexpr int64_t kGroupMaxSlots = 32;  // rows up to this many slots are packed several to a wave
 constexpr int64_t kTeamMinRows = 6;
 
@@ -304,10 +370,10 @@ constexpr int64_t kTeamMinRows = 6;
 // rows 131 / 220 us against 132 / 236 us for four; bf16 four rows 70 / 114 us against 101 / 146 us
 // for eight), fewer when the rows are too few to give every SIMD a few waves, but 4 bytes' worth at
 // least (bf16 100000 x 1024: two rows 135 / 234 us, one row 152 / 264 us).
-int kColumnRowsPerLane(int dtype, int64_t numseq) {
-  int v = 8 / elem_size_of(dtype);
-  const int least = 4 / elem_size_of(dtype);
-  while (v > least && numseq / v < 65536) v >>= 1;
+int kColumnRowsPerLane(const Problem& q) {
+  int v = 8 / elem_size_of(q.dtype);
+  const int least = 4 / elem_size_of(q.dtype);
+  while (v > least && q.numseq / v < q.at(65536)) v >>= 1;
   return v;
 }
 
@@ -320,7 +386,7 @@ int kColumnRowsPerLane(int dtype, int64_t numseq) {
 constexpr int64_t kSegmentBelowRows = 16384;
 constexpr int64_t kSegmentBelowRowsHalf = 32768;
 constexpr int64_t kSegmentMinLen = 256;       // shorter scan axes are left to the plain column kernels
-constexpr int64_t kSegmentWaves = 1024;       // waves a segmented launch aims for (one per SIMD)
+int64_t segment_waves(const Problem& q) { return 4 * q.cus; }  // waves a segmented launch aims for (one per SIMD)
 constexpr int64_t kSegmentMaxSegments = 4096; // (the maps of a row are then 32 KiB)
 
 size_t segment_maps_bytes(int64_t numseq, int64_t segments) { return size_t(2) * size_t(segments) * size_t(numseq) * 4; }
@@ -363,7 +429,7 @@ constexpr int64_t kColblockMinLen = 256;
 // 68 / 121 us against 71 / 128 us, 16384 x 4096 134 / 236 us against 145 / 254 us; 14000 x 2048 70 / 115 us
 // against 66 / 114 us, 16384 x 512 16 / 34 us against 19 / 31 us).
 bool colblock_full_house(const Problem& q) {
-  return q.dtype == LINREC_DTYPE_F32 && q.numseq >= 15360 && q.numseq <= 16384 && q.seqlen >= 1024 && q.row_stride == 1 &&
+  return q.dtype == LINREC_DTYPE_F32 && q.numseq >= q.at(15360) && q.numseq <= q.at(16384) && q.seqlen >= 1024 && q.row_stride == 1 &&
          q.col_phase % 2 == 0 && q.elem_stride % 2 == 0 && q.numseq % 2 == 0 &&
          (!q.batched() || (q.rows_per_batch % 2 == 0 && q.batch_stride % 2 == 0));
 }
@@ -380,23 +446,23 @@ int colblock_groups(const Problem& q) {
     // 12000 x 2048 68 us against 82 us, 16384 x 2048 73 us against 100 us); undivided waves beyond
     // (17408 x 2048 56 / 103 us against 72 / 124 us with two groups and 79 / 104 us for segments,
     // 32768 x 2048 70 / 123 us against 134 / 221 us for the plain kernel)
-    if (q.numseq >= (q.is_bwd ? 10240 : 8192) && q.numseq <= 16384) return 2;
-    return q.numseq > 16384 && q.numseq <= 65536 ? 1 : 0;
+    if (q.numseq >= q.at(q.is_bwd ? 10240 : 8192) && q.numseq <= q.at(16384)) return 2;
+    return q.numseq > q.at(16384) && q.numseq <= q.at(65536) ? 1 : 0;
   }
-  if (q.numseq >= (q.is_bwd ? 6144 : 4096) && q.numseq <= 8192) {
+  if (q.numseq >= q.at(q.is_bwd ? 6144 : 4096) && q.numseq <= q.at(8192)) {
     // two groups of 32 floats are 128-byte accesses: lines that do not start on a 128-byte boundary cost
     // them more than the undivided wave (7000 x 2048: 55 / 102 us against 50 / 86 us; 5000 x 2048 forward
     // 39 us against 47 us all the same)
-    if (q.numseq >= 6144 && (q.elem_stride * 4) % 128 != 0) return 1;
+    if (q.numseq >= q.at(6144) && (q.elem_stride * 4) % 128 != 0) return 1;
     return 2;
   }
   if (colblock_full_house(q)) return 2;
-  if (q.numseq > 8192 && q.numseq <= 32768) return 1;
+  if (q.numseq > q.at(8192) && q.numseq <= q.at(32768)) return 1;
   // Beyond one workgroup per CU the second round has to be at least half full to beat the plain kernel:
   // two rows per lane, 384 to 480 workgroups (50000 x 2048 246 / 421 us against 284 / 457 us, 57344 x 2048
   // 244 / 425 us against 272 / 457 us; 40000 x 2048 210 / 359 us against 174 / 314 us, 45056 x 2048
   // 216 / 381 us against 214 / 337 us, 65536 x 2048 271 / 487 us against 281 / 452 us)
-  return q.numseq >= 49152 && q.numseq <= 61440 ? 1 : 0;
+  return q.numseq >= q.at(49152) && q.numseq <= q.at(61440) ? 1 : 0;
 }
 // The block kernel for `vec` rows per lane with runs of `want_depth` positions, or of the compiled length
 // (8, or 4 where three tensors of two rows per lane would not fit the registers) for 0; -1 if none.
@@ -416,7 +482,7 @@ int colblock_rows_per_lane(const Problem& q, int want) {
   if (q.elem_stride == 1 && q.seqlen != 1) return 0;
   if (q.seqlen > 2147483647LL - 1024) return 0;  // positions are counted in 32 bits, a step beyond the row end included
   if (q.row_stride != 1 && q.numseq != 1 && q.rows_per_batch != 1) return 0;
-  int v = want > 0 ? want : q.dtype != LINREC_DTYPE_F32 ? 2 : (q.numseq > 16384 || colblock_full_house(q)) ? 2 : 1;
+  int v = want > 0 ? want : q.dtype != LINREC_DTYPE_F32 ? 2 : (q.numseq > q.at(16384) || colblock_full_house(q)) ? 2 : 1;
   auto fits = [&](int w) {
     return w == 1 || (q.row_stride == 1 && q.col_phase % w == 0 && q.elem_stride % w == 0 && q.numseq % w == 0 &&
                       (!q.batched() || (q.rows_per_batch % w == 0 && q.batch_stride % w == 0)));
@@ -495,11 +561,11 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       // tiling; with fewer than about a hundred rows the chip is not filled and look-back wins.
       if (q.base_mis >= 0 && full_slots > kLongRowSlots) {
         if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
-        else if (q.numseq >= kStreamMinRows) family = LINREC_FAMILY_STREAM;
+        else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) family = LINREC_FAMILY_STREAM;
         else if (q.numseq >= kTeamMinRows) family = LINREC_FAMILY_TEAM;
       }
     } else if (q.row_stride == 1 || q.numseq == 1 || q.rows_per_batch == 1) {
-      family = q.numseq < (half ? kSegmentBelowRowsHalf : kSegmentBelowRows) && q.seqlen >= kSegmentMinLen
+      family = q.numseq < q.at(half ? kSegmentBelowRowsHalf : kSegmentBelowRows) && q.seqlen >= kSegmentMinLen
                    ? LINREC_FAMILY_SEGMENT : LINREC_FAMILY_COLUMN;
       // a few thousand to a few ten thousand rows: workgroups whose waves share rows
       if (const int g = colblock_groups(q)) {
@@ -571,7 +637,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // (512 x 262144: 274 / 478 us against 282 / 491 us) or many (1024 x 65536 forward: 135.5 against
     // 138.7 us; 4096 x 65536: 542 against 556 us).  512 x 65536 is the same either way.
     const bool big_tiles = !half && rows_on_slots && q.seqlen % 16384 == 0 &&
-                           (q.numseq <= kComputeUnits || q.seqlen >= 131072 || (q.numseq >= 1024 && q.seqlen >= 32768));
+                           (q.numseq <= q.cus || q.seqlen >= 131072 || (q.numseq >= 4 * q.cus && q.seqlen >= 32768));
     // Tiles of 4096 elements for rows they pad less, and for rows of at most two of the larger tiles:
     // a partial last tile costs a whole one, and short walks overlap little (3355 x 10000: 73 / 122 us
     // against 77 / 162 us; 2500 x 14000 backward: 129 against 145 us; 1677 x 20000 backward: 126
@@ -592,8 +658,8 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // 94 / 159 us against 101 / 180 us.  With more rows in the last round, or more rounds, it brings
     // nothing (557 x 60164: 88 / 146 us against 91 / 149 us) or loses (389 x 86108: 87 / 147 us against
     // 83 / 139 us), because the second launch waits for the first.
-    if (!tune && q.numseq > kComputeUnits && q.numseq <= kComputeUnits + kTailMaxRows)
-      out->tail_rows = int32_t(q.numseq - kComputeUnits);
+    if (!tune && q.numseq > q.cus && q.numseq <= q.cus + q.at(kTailMaxRows))
+      out->tail_rows = int32_t(q.numseq - q.cus);
     size_t tail_workspace = 0;
     if (out->tail_rows) {
       linrec_plan_t tail;
@@ -621,10 +687,12 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     const int64_t tiles_per_row = q.seqlen / tile_elems;
     int64_t team = tune && tune->tasks > 0 ? tune->tasks : sweep_team_size(tiles_per_row);
     if (team > 64 || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
-    int64_t teams = tune && tune->carry > 0 ? tune->carry
-                                            : (q.is_bwd ? kSweepWorkgroupsBwd : kSweepWorkgroupsFwd) / team;
-    if (teams < 1) teams = 1;
+    // Every workgroup of the launch has to be resident at once (a walker waits for its team mates, and a
+    // workgroup that has not started yet only starts when another one ends): never more than the CUs hold.
+    const int64_t resident = int64_t(workgroups_per_cu(id, 64 * waves, q.is_bwd ? 1 : 2)) * q.cus;
+    int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
+    if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;
     if (q.numseq * tiles_per_row > 2147483647LL) return LINREC_E_TOO_LARGE;
     out->family = LINREC_FAMILY_SWEEP;
     out->waves = waves; out->slots = slots; out->vec = fv; out->carry = 1;
@@ -648,10 +716,12 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     const int id = find_kernel(q.dtype, LINREC_FAMILY_TEAM, waves, slots, fv, mode, desc, 1);
     if (id < 0) return LINREC_E_UNSUPPORTED;
     const int64_t tiles_per_row = ceil_div(full_slots, int64_t(waves) * slots * 64);
-    int64_t team = tune && tune->tasks > 0 ? tune->tasks : kTeamWorkgroups / q.numseq;
+    int64_t team = tune && tune->tasks > 0 ? tune->tasks : team_workgroups(q) / q.numseq;
     if (team < 2 && !(tune && tune->tasks > 0)) team = 2;
     if (team > tiles_per_row) team = tiles_per_row;
     if (team > 64) team = 64;  // one wave gathers the team's maps, one lane per team mate
+    // a team has to fit the chip, or its members would wait for mates that cannot start
+    if (team > int64_t(workgroups_per_cu(id, 64 * waves, 1)) * q.cus) return LINREC_E_UNSUPPORTED;
     if (q.numseq * team > 2147483647LL || q.numseq * tiles_per_row > 2147483647LL) return LINREC_E_TOO_LARGE;
     out->family = LINREC_FAMILY_TEAM;
     out->waves = waves; out->slots = slots; out->vec = fv; out->carry = 1;
@@ -693,7 +763,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       else if (max_slots <= 4096 && !half) { waves = 16; slots = 4; }
       else { waves = 8; slots = half ? 4 : 8; carry = 1; }
       // Few rows of a few thousand elements: split them so that the whole chip has work.
-      if (!carry && max_slots > 1024 && q.numseq < kSplitBelowRows) { waves = 4; slots = half ? 2 : 4; carry = 1; }
+      if (!carry && max_slots > 1024 && q.numseq < q.at(kSplitBelowRows)) { waves = 4; slots = half ? 2 : 4; carry = 1; }
     }
     if (tune && tune->family == LINREC_FAMILY_TILE) {
       if (tune->waves > 0) waves = tune->waves;
@@ -748,7 +818,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // Never more waves than the target: the waves beyond a whole number per SIMD would run alone at the
     // end (12288 x 4096, 96 waves per segment: 10 segments 174 / 268 us, 11 segments 193 / 287 us)
     const int64_t lanes = ceil_div(q.numseq, vec);
-    int64_t segments = given && tune->tasks > 0 ? tune->tasks : std::max<int64_t>(1, kSegmentWaves * 64 / lanes);
+    int64_t segments = given && tune->tasks > 0 ? tune->tasks : std::max<int64_t>(1, segment_waves(q) * 64 / lanes);
     if (segments > kSegmentMaxSegments) {
       if (given && tune->tasks > 0) return LINREC_E_UNSUPPORTED;
       segments = kSegmentMaxSegments;
@@ -795,12 +865,12 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
   if (family == LINREC_FAMILY_COLUMN && q.row_stride != 1 && q.numseq != 1 && q.rows_per_batch != 1) return LINREC_E_UNSUPPORTED;
   const bool depth_given = tune && tune->family == family && tune->slots > 0;
   const bool width_given = tune && tune->family == family && tune->waves > 0;
-  const int cap = family != LINREC_FAMILY_COLUMN ? 1 : width_given ? tune->waves : kColumnRowsPerLane(q.dtype, q.numseq);
+  const int cap = family != LINREC_FAMILY_COLUMN ? 1 : width_given ? tune->waves : kColumnRowsPerLane(q);
   // candidate access widths the layout allows: the preferred one first, then narrower, then wider
   // Timesteps in flight per lane: 8, or 16 when the launch has at most one wave per SIMD and each wave
   // has to keep more of the memory system busy (32768 x 2048: 145 / 254 us against 205 / 304 us;
   // 65536 x 1024 the same either way; 80000 x 1024: 174 / 317 us against 158 / 307 us).
-  const bool deep = ceil_div(ceil_div(q.numseq, cap), 64) <= 4 * kComputeUnits;
+  const bool deep = ceil_div(ceil_div(q.numseq, cap), 64) <= 4 * q.cus;
   int vec = 1, depth = depth_given ? tune->slots : 8, id = -1;
   for (int pass = 0; pass < 2 && id < 0; ++pass) {
     for (int v = pass == 0 ? cap : fv; v >= 1 && id < 0; v >>= 1) {
@@ -831,7 +901,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
   // 150000 x 256: 104.5 / 180.4 us against 87.7 / 158.2 us; 262144 x 256, 512 workgroups of four
   // waves: 132.5 / 223.8 us against 131.9 / 229.6 us).
   const int64_t lanes = ceil_div(q.numseq, vec);
-  const int block = lanes % (256 * kComputeUnits) == 0 ? 256 : 64;
+  const int block = lanes % (256 * q.cus) == 0 ? 256 : 64;
   out->grid = ceil_div(lanes, block);
   if (out->grid > 2147483647LL) return LINREC_E_TOO_LARGE;
   out->block = block;
@@ -977,6 +1047,19 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
   return e == hipSuccess ? int(hipGetLastError()) : int(e);
 }
 
+// The problem a forward call poses (misalignment of its pointers, device in hand).
+Problem forward_problem(int dtype, const void* inputs, const void* coeffs, const void* outputs, int64_t numseq,
+                        int64_t seqlen, int64_t row_stride, int64_t elem_stride, int64_t rows_per_batch,
+                        int64_t batch_stride, int reverse) {
+  const void* ptrs[] = {inputs, coeffs, outputs};
+  Problem q{numseq, seqlen, row_stride, elem_stride, reverse, 0, common_misalignment(ptrs, 3, dtype), false, dtype, 0,
+            rows_per_batch, batch_stride};
+  q.aligned16 = q.base_mis == 0;
+  q.col_phase = q.base_mis >= 0 ? q.base_mis : 1;
+  q.cus = compute_units();
+  return q;
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const linrec::v4f* __restrict__ src,
                                                    linrec::v4f* __restrict__ dst, long long n4) {
   // 4 slots per lane, 64-lane interleave: the access pattern of tile_kernel<4, 4, 4, ...>
@@ -1111,6 +1194,7 @@ int linrec_plan(int dtype, const void* any_input, int64_t numseq, int64_t seqlen
   Problem q{numseq, seqlen, row_stride, elem_stride, reverse, is_bwd, common_misalignment(ptrs, 1, dtype), false, dtype, 0};
   q.aligned16 = q.base_mis == 0;
   q.col_phase = q.base_mis >= 0 ? q.base_mis : 1;
+  q.cus = compute_units();
   return make_plan(q, tuning, plan);
 }
 
@@ -1126,6 +1210,7 @@ size_t linrec_workspace_bytes_dtype(int dtype, int64_t numseq, int64_t seqlen, i
   if (dtype < LINREC_DTYPE_F32 || dtype > LINREC_DTYPE_BF16) return 0;
   const int mis = align_elems < 0 ? -1 : align_elems & (full_vec_of(dtype) - 1);
   Problem q{numseq, seqlen, row_stride, elem_stride, 0, is_bwd, mis, mis == 0, dtype, mis >= 0 ? mis : 1};
+  q.cus = compute_units();
   linrec_plan_t plan;
   if (make_plan(q, tuning, &plan) != LINREC_OK) return 0;
   return size_t(plan.workspace_bytes);
@@ -1145,11 +1230,8 @@ int fwd_impl(int dtype, const void* inputs, const void* coeffs, void* outputs, i
   if (dtype < LINREC_DTYPE_F32 || dtype > LINREC_DTYPE_BF16) return LINREC_E_UNSUPPORTED;
   if (numseq == 0 || seqlen == 0) return LINREC_OK;
   if (!inputs || !coeffs || !outputs) return LINREC_E_INVALID;
-  const void* ptrs[] = {inputs, coeffs, outputs};
-  Problem q{numseq, seqlen, row_stride, elem_stride, reverse, 0, common_misalignment(ptrs, 3, dtype), false, dtype, 0,
-            rows_per_batch, batch_stride};
-  q.aligned16 = q.base_mis == 0;
-  q.col_phase = q.base_mis >= 0 ? q.base_mis : 1;
+  const Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride,
+                                    rows_per_batch, batch_stride, reverse);
   linrec_plan_t plan;
   int rc = make_plan(q, tuning, &plan);
   if (rc != LINREC_OK) return rc;
@@ -1179,6 +1261,7 @@ int bwd_impl(int dtype, const void* d_outputs, const void* coeffs, const void* o
             rows_per_batch, batch_stride};
   q.aligned16 = q.base_mis == 0;
   q.col_phase = q.base_mis >= 0 ? q.base_mis : 1;
+  q.cus = compute_units();
   linrec_plan_t plan;
   int rc = make_plan(q, tuning, &plan);
   if (rc != LINREC_OK) return rc;
@@ -1240,6 +1323,7 @@ int linrec_plan_batched(int dtype, const void* any_input, int64_t batches, int64
             common_misalignment(ptrs, 1, dtype), false, dtype, 0, rows_per_batch, batch_stride};
   q.aligned16 = q.base_mis == 0;
   q.col_phase = q.base_mis >= 0 ? q.base_mis : 1;
+  q.cus = compute_units();
   return make_plan(q, tuning, plan);
 }
 
@@ -1258,6 +1342,14 @@ int linrec_bwd_f32(const float* d_outputs, const float* coeffs, const float* out
   return linrec_bwd(LINREC_DTYPE_F32, d_outputs, coeffs, outputs, d_inputs, d_coeffs, numseq, seqlen, row_stride,
                     elem_stride, reverse, workspace, workspace_bytes, tuning, stream);
 }
+
+int linrec_set_compute_units(int cus) {
+  const int old = g_cu_override.load(std::memory_order_relaxed);
+  if (cus >= 0) g_cu_override.store(cus, std::memory_order_relaxed);
+  return old;
+}
+
+int linrec_compute_units(void) { return compute_units(); }
 
 int linrec_set_spin_limit(int polls) {
   const int old = g_spin_limit;

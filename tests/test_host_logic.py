@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "linrec_hip.h")).read()
     declared = set(re.findall(r"^\s*(?:int|size_t|const char\*|void)\s+(linrec_\w+)\s*\(", header, flags=re.M))
-    assert len(declared) == 25, declared
+    assert len(declared) == 27, declared
     lib = ctypes.CDLL(nat.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/linrec_hip.h but not exported"
@@ -37,6 +37,46 @@ def test_error_strings():
         nat.check(-3, "x")
     with pytest.raises(RuntimeError):
         nat.check(-1, "x")
+
+
+def test_planner_follows_the_compute_unit_count():
+    """Grids of the kernels whose workgroups wait for each other are sized by the device's CU count
+    (asked once per device; 256 assumed on a host without one), never by a constant."""
+    lib = nat.lib()
+    assert lib.linrec_set_compute_units(-1) == 0  # no override in force
+    if not torch.cuda.is_available():
+        assert lib.linrec_compute_units() == 256
+    x = torch.empty(16, 1048576)
+    try:
+        seen = {}
+        for cus in (256, 128, 64, 20):
+            lib.linrec_set_compute_units(cus)
+            assert lib.linrec_compute_units() == cus
+            for is_bwd in (False, True):
+                p = nat.plan(x, False, is_bwd)
+                if cus == 20:  # 16 rows are "many" for 20 CUs: one workgroup per row, nobody waits
+                    assert p["family"] == nat.FAMILY_STREAM and p["workspace_bytes"] == 0
+                    continue
+                assert p["family"] == nat.FAMILY_SWEEP
+                # forward: at most two workgroups per CU, backward one; whole teams only
+                assert p["grid"] <= (1 if is_bwd else 2) * cus and p["grid"] % p["tasks"] == 0
+                seen[(cus, is_bwd)] = p["grid"]
+            # one team of workgroups per row: never more workgroups than CUs
+            t = nat.plan(torch.empty(8, 1048580), False, False)
+            assert t["family"] == nat.FAMILY_TEAM and t["grid"] <= cus and t["tasks"] == cus // 8
+            # one workgroup per row from half the CUs on, teams below
+            assert nat.plan(torch.empty(cus // 2 + 1, 65540))["family"] == nat.FAMILY_STREAM
+            assert nat.plan(torch.empty(cus // 2, 65540))["family"] == nat.FAMILY_TEAM
+        assert seen[(256, False)] == 256 and seen[(128, False)] == 256 and seen[(64, False)] == 128
+        assert seen[(256, True)] == 256 and seen[(128, True)] == 128 and seen[(64, True)] == 64
+        # a team that cannot be resident at once is refused rather than left to wait for absent mates
+        lib.linrec_set_compute_units(8)
+        with pytest.raises(NotImplementedError):
+            nat.plan(x, False, True, nat.Tuning(nat.FAMILY_SWEEP, 8, 4, 4, 16))
+        with pytest.raises(NotImplementedError):
+            nat.plan(torch.empty(2, 1048580), False, False, nat.Tuning(nat.FAMILY_TEAM, 8, 4, -1, 16))
+    finally:
+        lib.linrec_set_compute_units(0)
 
 
 def _plan(shape, reverse=False, is_bwd=False, tuning=None, strides=None):
