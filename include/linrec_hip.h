@@ -32,6 +32,7 @@ extern "C" {
 #define LINREC_E_WORKSPACE (-2)   /* workspace missing, misaligned or too small for this call */
 #define LINREC_E_UNSUPPORTED (-3) /* tuning override names a kernel that is not compiled in */
 #define LINREC_E_TOO_LARGE (-4)   /* seqlen beyond 2^31-5 elements */
+#define LINREC_E_SCRATCH (-5)     /* linrec_fwd_noalloc: the call needs more scratch than the static array holds */
 
 /* Storage types (arithmetic is always fp32). */
 #define LINREC_DTYPE_F32 0
@@ -144,6 +145,28 @@ int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void*
                void* d_coeffs, int64_t numseq, int64_t seqlen, int64_t row_stride, int64_t elem_stride,
                int reverse, void* workspace, size_t workspace_bytes, const linrec_tuning_t* tuning,
                void* stream);
+
+/*
+ * linrec_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same call without the workspace arguments.
+ * It has no counterpart in the reference, whose launcher allocates its result itself
+ * (linrec/impl/cuda/linrec_pipe.cu:31).  Where the chosen kernel needs a workspace, the library's own
+ * static device array of LINREC_NOALLOC_SCRATCH_BYTES serves as one; each GPU holds its copy of that
+ * array from the first call on it until the process ends.  The call makes no hipMalloc / hipFree and
+ * calls no allocating routine.  A problem that needs more than the array holds (about 130 000 tiles of
+ * rows split over workgroups) returns LINREC_E_SCRATCH with nothing enqueued; results are identical to
+ * linrec_fwd's.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (two streams, two threads) race on it and must be serialised by the caller, and the array must not
+ * be mixed with linrec_fwd's caller-owned workspaces in any other way than by calling this function.
+ * The array keeps the previous call's contents; nothing in it needs clearing between calls (its launch
+ * counter tells old descriptors from new ones, and the completion counters end every launch at zero).
+ * The first call on a device looks up the array's address there (hipGetSymbolAddress); make that call
+ * outside graph capture.
+ */
+#define LINREC_NOALLOC_SCRATCH_BYTES (4u << 20)
+int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t numseq,
+                       int64_t seqlen, int64_t row_stride, int64_t elem_stride, int reverse,
+                       const linrec_tuning_t* tuning, void* stream);
 
 /*
  * Batches of matrices whose scan axis is the strided one, e.g. (batch, time, channels) tensors

@@ -80,6 +80,7 @@ def _declare(lib):
         "linrec_set_spin_limit": (i32, [i32]),
         "linrec_compute_units": (i32, []),
         "linrec_set_compute_units": (i32, [i32]),
+        "linrec_fwd_noalloc": (i32, [i32, p, p, p, i64, i64, i64, i64, i32, tun, p]),
         "linrec_kernel_count": (i32, []),
         "linrec_kernel_name": (ctypes.c_char_p, [i32]),
         "linrec_kernel_attrs": (i32, [i32] + [ctypes.POINTER(ctypes.c_int)] * 4),

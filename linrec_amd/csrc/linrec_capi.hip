@@ -21,6 +21,15 @@
 #include "team_kernel.hpp"
 #include "tile_kernel.hpp"
 
+// Scratch of linrec_fwd_noalloc, the entry point for callers that cannot allocate: every GPU the library
+// runs on holds one copy of this array, at its own address, until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress (device_state() below keeps the address per device);
+// kernels and copies are given that address, never the name.  It starts out zero-filled, which is the
+// state a look-back workspace has to be in before its first launch, and every launch leaves it usable
+// for the next (the counters end at zero, the launch counter moves on).
+constexpr size_t kStaticScratchBytes = LINREC_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 using linrec::ColumnArgs;
@@ -207,14 +216,16 @@ int find_kernel(int dtype, int family, int waves, int slots, int vec, int mode, 
 // ---- the device ------------------------------------------------------------------------------
 // What the planner needs to know about the device a call runs on, asked once per device (the
 // reference asks through cudaDeviceGetAttribute, linrec/impl/cuda/cuhelpers.cuh:23-34, on every
-// launch, linrec_pipe.cu:72-80): the number of compute units and how many workgroups of a kernel one CU
-// holds.
+// launch, linrec_pipe.cu:72-80): the number of compute units, how many workgroups of a kernel one CU
+// holds, and where this device keeps its copy of the static scratch array.
 constexpr int kDefaultComputeUnits = 256;  // MI355X; assumed when a plan is asked for on a host without a GPU
 constexpr int kMaxDevices = 64;
 
 struct DeviceState {
   std::once_flag once;
   int cus = 0;                  // hipDeviceAttributeMultiprocessorCount
+  void* scratch_ptr = nullptr;  // this device's address of `scratch`
+  int scratch_rc = -1;          // hipError_t of the hipGetSymbolAddress call that produced it
   std::mutex occupancy_mutex;
   std::vector<int8_t> occupancy;  // per kernel id: workgroups one CU holds, 0 = not asked yet
 };
@@ -234,6 +245,11 @@ DeviceState* device_state() {
     int n = 0;
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) d.cus = n;
     else (void)hipGetLastError();
+    d.scratch_rc = int(hipGetSymbolAddress(&d.scratch_ptr, HIP_SYMBOL(scratch)));
+    if (d.scratch_rc != 0) {
+      (void)hipGetLastError();
+      d.scratch_ptr = nullptr;
+    }
   });
   return &d;
 }
@@ -1174,6 +1190,7 @@ const char* linrec_hip_error_string(int code) {
     case LINREC_E_WORKSPACE: return "linrec: workspace missing, not 16-byte aligned or too small";
     case LINREC_E_UNSUPPORTED: return "linrec: no compiled kernel matches the requested tuning/layout";
     case LINREC_E_TOO_LARGE: return "linrec: problem too large (seqlen or tile count beyond 2^31)";
+    case LINREC_E_SCRATCH: return "linrec: the call needs more scratch than the library's static 4 MiB array holds";
     default: return code > 0 ? hipGetErrorString(hipError_t(code)) : "linrec: unknown error";
   }
 }
@@ -1285,6 +1302,31 @@ int linrec_fwd(int dtype, const void* inputs, const void* coeffs, void* outputs,
                size_t workspace_bytes, const linrec_tuning_t* tuning, void* stream) {
   return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, workspace,
                   workspace_bytes, tuning, stream);
+}
+
+int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t numseq,
+                       int64_t seqlen, int64_t row_stride, int64_t elem_stride, int reverse,
+                       const linrec_tuning_t* tuning, void* stream) {
+  if (numseq < 0 || seqlen < 0) return LINREC_E_INVALID;
+  if (dtype < LINREC_DTYPE_F32 || dtype > LINREC_DTYPE_BF16) return LINREC_E_UNSUPPORTED;
+  if (numseq == 0 || seqlen == 0) return LINREC_OK;
+  if (!inputs || !coeffs || !outputs) return LINREC_E_INVALID;
+  // What the call needs follows from its arguments alone, so a call that needs more than the static
+  // array holds is turned down before anything is enqueued.
+  const Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse);
+  linrec_plan_t plan;
+  const int rc = make_plan(q, tuning, &plan);
+  if (rc != LINREC_OK) return rc;
+  if (plan.workspace_bytes > kStaticScratchBytes) return LINREC_E_SCRATCH;
+  if (plan.workspace_bytes == 0)
+    return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, nullptr, 0,
+                    tuning, stream);
+  DeviceState* d = device_state();
+  if (!d) return int(hipErrorNoDevice);
+  if (!d->scratch_ptr) return d->scratch_rc > 0 ? d->scratch_rc : int(hipErrorInvalidSymbol);
+  // The array's size is always passed whole: the split into counters and descriptors depends on it.
+  return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, d->scratch_ptr,
+                  kStaticScratchBytes, tuning, stream);
 }
 
 int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void* outputs, void* d_inputs,

@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "linrec_hip.h")).read()
     declared = set(re.findall(r"^\s*(?:int|size_t|const char\*|void)\s+(linrec_\w+)\s*\(", header, flags=re.M))
-    assert len(declared) == 27, declared
+    assert len(declared) == 28, declared
     lib = ctypes.CDLL(nat.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/linrec_hip.h but not exported"
@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_error_strings():
     lib = nat.lib()
-    for code in (0, -1, -2, -3, -4):
+    for code in (0, -1, -2, -3, -4, -5):
         assert lib.linrec_hip_error_string(code)
     with pytest.raises(NotImplementedError):
         nat.check(-3, "x")
@@ -77,6 +77,24 @@ def test_planner_follows_the_compute_unit_count():
             nat.plan(torch.empty(2, 1048580), False, False, nat.Tuning(nat.FAMILY_TEAM, 8, 4, -1, 16))
     finally:
         lib.linrec_set_compute_units(0)
+
+
+def test_noalloc_entry_point_rejects_what_its_static_scratch_cannot_hold():
+    """linrec_fwd_noalloc turns a call down, before anything touches a device, when the launch would need
+    more workspace than the library's static array (no pointer is dereferenced on the host)."""
+    lib = nat.lib()
+    fake = ctypes.c_void_p(1 << 20)
+    limit = 4 << 20
+    # one row of 2^31 - 8 floats: look-back tiles of 16384 elements, 131072 descriptors
+    n = (1 << 31) - 8
+    need = lib.linrec_workspace_bytes_dtype(0, 1, n, n, 1, 0, 0, None)
+    assert need > limit
+    assert lib.linrec_fwd_noalloc(0, fake, fake, fake, 1, n, n, 1, 0, None, None) == -5
+    assert b"scratch" in lib.linrec_hip_error_string(-5)
+    # invalid arguments are reported as by linrec_fwd
+    assert lib.linrec_fwd_noalloc(0, None, fake, fake, 4, 100000, 100000, 1, 0, None, None) == -1
+    assert lib.linrec_fwd_noalloc(7, fake, fake, fake, 4, 100000, 100000, 1, 0, None, None) == -3
+    assert lib.linrec_fwd_noalloc(0, fake, fake, fake, 0, 100000, 100000, 1, 0, None, None) == 0
 
 
 def _plan(shape, reverse=False, is_bwd=False, tuning=None, strides=None):

@@ -1,0 +1,82 @@
+"""GPU test of linrec_fwd_noalloc, the entry point for callers that cannot allocate device memory: through
+the C ABI its results must equal linrec_fwd's bit for bit (same kernels, the library's static scratch
+array in place of a caller-owned workspace), call after call on the same GPU, also when a later call is
+smaller than the one before and so finds the previous call's descriptors in the array."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from linrec_amd import _native as nat
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(shape, seed, transposed=False):
+    g = torch.Generator().manual_seed(seed)
+    if transposed:
+        x = torch.randn(shape[::-1], generator=g).cuda().t()
+        c = torch.rand(shape[::-1], generator=g).cuda().t()
+    else:
+        x = torch.randn(shape, generator=g).cuda()
+        c = torch.rand(shape, generator=g).cuda()
+    return x, c
+
+
+def _both(x, c, reverse):
+    """(result of linrec_fwd with a workspace of its own, result of linrec_fwd_noalloc)"""
+    lib = nat.lib()
+    lay = nat.row_layout(x)
+    assert lay is not None
+    stream = torch.cuda.current_stream().cuda_stream
+    want = torch.full_like(x, float("nan"))
+    got = torch.full_like(x, float("nan"))
+    need = lib.linrec_workspace_bytes_dtype(nat.DTYPES[x.dtype], *lay, 0, 0, None)
+    ws = torch.zeros(max(need, 16), dtype=torch.uint8, device=x.device)
+    rc = lib.linrec_fwd(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), want.data_ptr(), *lay, int(reverse),
+                        ws.data_ptr(), ws.numel(), None, stream)
+    assert rc == 0, rc
+    rc = lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, int(reverse),
+                                None, stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    return want, got, need
+
+
+def test_noalloc_forward_equals_forward_with_a_workspace_call_after_call():
+    # each of these launches keeps state in the scratch: teams that go from row to row (16 rows), look-back
+    # tiles (3 rows, then 1 row), one team per row (8 ragged rows), segments of a strided scan axis
+    cases = [((16, 131072), False, False), ((3, 40000), True, False), ((1, 9000), False, False),
+             ((8, 70001), False, False), ((16, 65536), True, False), ((1024, 4096), False, True),
+             ((2, 20000), False, False)]
+    used_scratch = 0
+    for i, (shape, reverse, transposed) in enumerate(cases):
+        print("noalloc case", i, shape, reverse, transposed, flush=True)
+        x, c = _pair(shape, 100 + i, transposed)
+        want, got, need = _both(x, c, reverse)
+        used_scratch += need > 0
+        assert not torch.isnan(got).any()
+        assert torch.equal(want, got), (shape, (want - got).abs().max().item())
+    assert used_scratch >= 6
+    # the small last case also against the float64 recurrence (bar: 1e-5 normwise, as everywhere)
+    truth = oracle.fwd(x.cpu().numpy(), c.cpu().numpy(), False, dtype=np.float64)
+    assert oracle.error_report(got.cpu().numpy(), truth)["normwise"] <= 1e-5
+    assert nat.gave_up_count() == 0
+
+
+def test_noalloc_forward_of_16_bit_storage_and_kernels_without_scratch():
+    lib = nat.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    for dtype, shape in ((torch.bfloat16, (16, 131072)), (torch.float16, (4, 50000)), (torch.float32, (64, 4096))):
+        g = torch.Generator().manual_seed(7)
+        x = torch.randn(shape, generator=g).to(dtype).cuda()
+        c = torch.rand(shape, generator=g).to(dtype).cuda()
+        lay = nat.row_layout(x)
+        got = torch.full_like(x, float("nan"))
+        assert lib.linrec_fwd_noalloc(nat.DTYPES[dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0, None,
+                                      stream) == 0
+        want = nat.fwd(x, c)
+        torch.cuda.synchronize()
+        assert torch.equal(want, got), (dtype, shape)
