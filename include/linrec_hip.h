@@ -65,6 +65,10 @@ extern "C" {
                                   starts by the unused coefficient there.  Tuning: `slots` = rows of 64 slots
                                   a wave takes (4 or 2) */
 
+#define LINREC_FAMILY_DRIFT 10  /* the SWEEP launch shape with the exchange between team mates off the critical
+                                  path: a scanned tile is kept in registers and stored two steps late, by which
+                                  time the value entering it has arrived without anybody waiting.  Tuning as SWEEP */
+
 /*
  * Per-call tuning override; NULL selects the built-in gfx950 table.
  * Replaces the keyword options of the reference's launchers

@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "liblinrec_hip.so")
 FAMILY_AUTO, FAMILY_TILE, FAMILY_COLUMN, FAMILY_NAIVE, FAMILY_STREAM, FAMILY_TEAM, FAMILY_SWEEP, FAMILY_GROUP = 0, 1, 2, 3, 4, 5, 6, 7
 FAMILY_SEGMENT = 8
 FAMILY_FLAT = 9
+FAMILY_DRIFT = 10
 
 
 DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}  # LINREC_DTYPE_*

@@ -75,10 +75,10 @@ __global__ __launch_bounds__(64 * NW) void chain_kernel(TileArgs p) {
       sh_b[wave] = r.total.b;
     }
     __syncthreads();
-    const Affine before = fold_waves<NW>(sh_a, sh_b, wave);
+    Affine before, total;
+    wave_prefixes<NW>(sh_a, sh_b, wave, lane, before, total);
     if (wave == 0) {
       uint64_t* desc = p.desc + 2 * (t.row * p.tiles_per_row);
-      const Affine total = fold_waves<NW>(sh_a, sh_b, NW);
       float carry_in = 0.0f;
       if (k == 0) {
         if (lane == 0) st_desc(desc + 1, pack_desc((seq << 2) | STATUS_INCLUSIVE, total.b));
@@ -87,7 +87,9 @@ __global__ __launch_bounds__(64 * NW) void chain_kernel(TileArgs p) {
           st_desc(desc + 2 * k, pack_desc((seq << 2) | STATUS_AGGREGATE, total.a));
           st_desc(desc + 2 * k + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, total.b));
         }
-        carry_in = look_back(desc, k, seq, lane, p.spin_limit, p.ws);
+        bool ok;
+        carry_in = look_back(desc, k, seq, lane, p.spin_limit, p.ws, ok);
+        if (!ok) carry_in = recompute_entry<VEC, MODE, DESC>(t.q, t.rv, k * TILE_SLOTS, lane);
         if (lane == 0)
           st_desc(desc + 2 * k + 1, pack_desc((seq << 2) | STATUS_INCLUSIVE, fmaf(carry_in, total.a, total.b)));
       }

@@ -14,6 +14,7 @@
 #include "colblock_kernel.hpp"
 #include "column_kernel.hpp"
 #include "flat_kernel.hpp"
+#include "drift_kernel.hpp"
 #include "group_kernel.hpp"
 #include "chain_kernel.hpp"
 #include "stream_kernel.hpp"
@@ -75,6 +76,14 @@ struct KernelEntry {
 #define SWEEP_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
+#define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
+  {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, 2>, DT, LINREC_FAMILY_DRIFT, \
+   NW, S, VEC, linrec::MODE, DESC, 1}
+#define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
+  DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
+#define DRIFT_BWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
+  DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
 #define TEAM_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                 \
   TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
 #define STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                      \
@@ -138,6 +147,8 @@ struct KernelEntry {
 #define CHAIN_(...) CHAIN_ALL_DIRS(__VA_ARGS__)
 #define TEAM_(...) TEAM_ALL_DIRS(__VA_ARGS__)
 #define SWEEP_(...) SWEEP_ALL_DIRS(__VA_ARGS__)
+#define DRIFT_FWD_(...) DRIFT_FWD_DIRS(__VA_ARGS__)
+#define DRIFT_BWD_(...) DRIFT_BWD_DIRS(__VA_ARGS__)
 #define TEAM_FWD_(...) TEAM_FWD_DIRS(__VA_ARGS__)
 #define STREAM_(...) STREAM_ALL_DIRS(__VA_ARGS__)
 #define COLUMN_(...) COLUMN_ALL_DIRS(__VA_ARGS__)
@@ -180,6 +191,8 @@ const KernelEntry kKernels[] = {
     TEAM_(F32, 4, 2, 4), TEAM_(F32, 4, 4, 4), TEAM_(F32, 8, 2, 4), TEAM_(F32, 8, 4, 4),
     // teams that go on from row to row so that the launch reads the tensors front to back
     SWEEP_(F32, 8, 4, 4), SWEEP_(F32, 8, 2, 4), SWEEP_(F32, 4, 4, 4), SWEEP_(F32, 8, 8, 4),
+    // the same launch shape with a tile stored two steps late, so that nobody waits for the exchange
+    DRIFT_FWD_(F32, 8, 4, 4), DRIFT_FWD_(F32, 8, 2, 4), DRIFT_BWD_(F32, 8, 2, 4), DRIFT_FWD_(F32, 4, 4, 4),
     // short rows: several rows per wave
     GROUP_(F32, 4),
     // short rows that are not whole slots, dense: the tensor as one flat array
@@ -204,7 +217,7 @@ int find_kernel(int dtype, int family, int waves, int slots, int vec, int mode, 
   for (int i = 0; i < kNumKernels; ++i) {
     const KernelEntry& k = kKernels[i];
     const bool waves_matter = family == LINREC_FAMILY_TILE || family == LINREC_FAMILY_STREAM ||
-                              family == LINREC_FAMILY_TEAM || family == LINREC_FAMILY_SWEEP || family == LINREC_FAMILY_GROUP ||
+                              family == LINREC_FAMILY_TEAM || family == LINREC_FAMILY_SWEEP || family == LINREC_FAMILY_DRIFT || family == LINREC_FAMILY_GROUP ||
                               family == LINREC_FAMILY_FLAT;
     if (k.dtype == dtype && k.family == family && k.slots == slots && k.vec == vec && k.mode == mode &&
         k.desc == desc && k.carry == carry && (!waves_matter || k.waves == waves))
@@ -303,8 +316,6 @@ int full_vec_of(int dtype) { return 16 / elem_size_of(dtype); }
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// Workgroups wanted in flight before splitting rows further stops paying: a few per CU.
-constexpr int64_t kEnoughWorkgroups = 1024;
 // Stream kernels take over from tiles for rows of more than 2048 slots once there are enough rows
 // to give every CU work.
 constexpr int64_t kLongRowSlots = 2048;  // 8192 floats, 16384 halves
@@ -328,11 +339,39 @@ constexpr int64_t kSweepMinTiles = 4;  // tiles per row below which the exchange
 // Team kernels: one workgroup per CU.
 int64_t team_workgroups(const Problem& q) { return q.cus; }
 
-// Largest divisor of `tiles_per_row` that is at most kSweepMaxTeam.
-int64_t sweep_team_size(int64_t tiles_per_row) {
-  for (int64_t m = kSweepMaxTeam; m > 1; --m)
+// Largest divisor of `tiles_per_row` that is at most `most`.
+int64_t sweep_team_size(int64_t tiles_per_row, int64_t most = kSweepMaxTeam) {
+  for (int64_t m = most; m > 1; --m)
     if (tiles_per_row % m == 0) return m;
   return 1;
+}
+
+// Drift kernels (fp32): the sweep launch shape without the wait for the exchange.  Measured against the
+// table's previous choice, forward / backward in us: 512 x 65536 67.9 / 113.3 against 70.7 (stream) / 120.7
+// (sweep); 288 x 65536 40.2 / 65.6 against 44.3 / 68.1; 1024 x 65536 132.5 / 224.8 against 138.0 / 233.0;
+// 1024 x 32768 68.3 / 114.0 against 72.9 / 118.8; 2048 x 16384 69.1 / 114.4 against 70.4 / 120.2;
+// 160 x 131072 44.8 / 73.8 against 47.9 / 78.5; 128 x 262144 69.4 / 116.3 against 78.7 / 119.9;
+// forward only: 16 x 1048576 40.3 against 43.5, 64 x 524288 70.0 against 78.0, 32 x 1048576 72.9 against
+// 81.9, 8 x 4194304 75.9 against 84.6, 512 x 262144 260.9 against 279.1.  Left to the others: more than
+// 2048 rows (4096 x 65536 553 / 959 against 548 / 948), and the backward of fewer than 128 rows or of rows
+// longer than 131072 (16 x 1048576 64.4 against 62.0, 64 x 524288 118.9 against 115.3, 512 x 262144 459.7
+// against 450.8), which tiles of 16384 elements serve better and a drift kernel has no registers for.
+// Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
+int drift_slots_for(const Problem& q, int fv) {
+  if (q.dtype != LINREC_DTYPE_F32) return 0;
+  if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
+  if (q.numseq * 64 < q.cus) return 0;  // teams of at most 64 would leave most of the chip idle
+  if (q.numseq > q.at(2048)) return 0;
+  if (q.is_bwd && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
+  for (int s : {4, 2}) {
+    if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
+    const int64_t tile = int64_t(8) * s * 64 * fv;
+    if (q.seqlen % tile != 0) continue;
+    const int64_t tiles_per_row = q.seqlen / tile;
+    if (tiles_per_row < kSweepMinTiles || sweep_team_size(tiles_per_row, 64) < kSweepMinTiles) continue;
+    return s;
+  }
+  return 0;
 }
 
 // Rows longer than a tile, every tile a full one: the sweep kernels spread any number of rows
@@ -576,7 +615,8 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       // MI355X at 2^25 elements: 512 x 65536 forward 71 us against 84 us for the best look-back
       // tiling; with fewer than about a hundred rows the chip is not filled and look-back wins.
       if (q.base_mis >= 0 && full_slots > kLongRowSlots) {
-        if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
+        if (drift_slots_for(q, fv) > 0) family = LINREC_FAMILY_DRIFT;
+        else if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
         else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) family = LINREC_FAMILY_STREAM;
         else if (q.numseq >= kTeamMinRows) family = LINREC_FAMILY_TEAM;
       }
@@ -689,33 +729,39 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     return LINREC_OK;
   }
 
-  if (family == LINREC_FAMILY_SWEEP) {
+  if (family == LINREC_FAMILY_SWEEP || family == LINREC_FAMILY_DRIFT) {
+    const bool drift = family == LINREC_FAMILY_DRIFT;
     if (q.elem_stride != 1 && q.seqlen != 1) return LINREC_E_UNSUPPORTED;
     if (q.numseq > 1 && q.row_stride < q.seqlen && q.row_stride > -q.seqlen) return LINREC_E_INVALID;
     const int waves = tune && tune->waves > 0 ? tune->waves : 8;
-    const int auto_slots = tune && tune->family == LINREC_FAMILY_SWEEP ? 0 : sweep_slots_for(q, fv);
+    const int auto_slots = tune && tune->family != LINREC_FAMILY_AUTO ? 0 : drift ? drift_slots_for(q, fv) : sweep_slots_for(q, fv);
     const int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? 2 : 4);
     const int64_t tile_elems = int64_t(waves) * slots * 64 * fv;
     // every tile of every row has to be a full one
     if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.seqlen % tile_elems != 0) return LINREC_E_UNSUPPORTED;
-    const int id = find_kernel(q.dtype, LINREC_FAMILY_SWEEP, waves, slots, fv, mode, desc, 1);
+    const int id = find_kernel(q.dtype, family, waves, slots, fv, mode, desc, 1);
     if (id < 0) return LINREC_E_UNSUPPORTED;
+    const int block = 64 * waves;
     const int64_t tiles_per_row = q.seqlen / tile_elems;
-    int64_t team = tune && tune->tasks > 0 ? tune->tasks : sweep_team_size(tiles_per_row);
-    if (team > 64 || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
     // Every workgroup of the launch has to be resident at once (a walker waits for its team mates, and a
     // workgroup that has not started yet only starts when another one ends): never more than the CUs hold.
-    const int64_t resident = int64_t(workgroups_per_cu(id, 64 * waves, q.is_bwd ? 1 : 2)) * q.cus;
+    const int64_t resident = int64_t(workgroups_per_cu(id, block, drift || q.is_bwd ? 1 : 2)) * q.cus;
+    // Drift kernels: as much of a row in flight at once as a team can hold (one wave collects a tile's
+    // maps, a lane per team mate: 64 at most), so that the launch's reading positions leave no gaps.
+    const int64_t team = tune && tune->tasks > 0
+                             ? tune->tasks
+                             : sweep_team_size(tiles_per_row, std::min<int64_t>(drift ? 64 : kSweepMaxTeam, resident));
+    if (team > 64 || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
     int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
     if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;
     if (q.numseq * tiles_per_row > 2147483647LL) return LINREC_E_TOO_LARGE;
-    out->family = LINREC_FAMILY_SWEEP;
+    out->family = family;
     out->waves = waves; out->slots = slots; out->vec = fv; out->carry = 1;
     out->tiles_per_row = int32_t(tiles_per_row);
     out->tasks = int32_t(team);
     out->grid = teams * team;
-    out->block = 64 * waves;
+    out->block = block;
     out->kernel_id = id;
     out->workspace_bytes = linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row);
     return LINREC_OK;
@@ -978,7 +1024,7 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
   if (plan.kernel_id < 0) return LINREC_OK;  // empty problem
   const KernelEntry& k = kKernels[plan.kernel_id];
   if (plan.family == LINREC_FAMILY_TILE || plan.family == LINREC_FAMILY_STREAM || plan.family == LINREC_FAMILY_TEAM ||
-      plan.family == LINREC_FAMILY_SWEEP) {
+      plan.family == LINREC_FAMILY_SWEEP || plan.family == LINREC_FAMILY_DRIFT) {
     if (plan.carry) {
       if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) || workspace_bytes < plan.workspace_bytes)
         return LINREC_E_WORKSPACE;
@@ -993,7 +1039,8 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
     a.numseq = q.numseq;
     a.tasks = plan.tasks > 0 ? plan.tasks : 1;
     a.row_groups = plan.family == LINREC_FAMILY_TEAM ? q.numseq
-                   : plan.family == LINREC_FAMILY_SWEEP ? plan.grid / a.tasks : ceil_div(q.numseq, a.tasks);
+                   : plan.family == LINREC_FAMILY_SWEEP || plan.family == LINREC_FAMILY_DRIFT ? plan.grid / a.tasks
+                                                                                              : ceil_div(q.numseq, a.tasks);
     a.ws = static_cast<linrec::CarryHeader*>(workspace);
     a.counters = nullptr; a.desc = nullptr; a.ws_tiles = 0;
     if (plan.carry) {

@@ -28,6 +28,10 @@ __device__ __forceinline__ float dpp_move(float old, float src) {
                                          CTRL, ROW_MASK, 0xf, false));
 }
 
+constexpr int DPP_ROW_SHL1 = 0x101;  // lane i <- lane i+1 of the same 16-lane row
+constexpr int DPP_ROW_SHL2 = 0x102;
+constexpr int DPP_ROW_SHL4 = 0x104;
+constexpr int DPP_ROW_SHL8 = 0x108;
 constexpr int DPP_ROW_SHR1 = 0x111;
 constexpr int DPP_ROW_SHR2 = 0x112;
 constexpr int DPP_ROW_SHR4 = 0x114;

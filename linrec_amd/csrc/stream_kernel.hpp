@@ -72,8 +72,8 @@ __global__ __launch_bounds__(64 * NW) void stream_kernel(TileArgs p) {
       sh_b[par][wave] = r.total.b;
     }
     __syncthreads();
-    const Affine before = fold_waves<NW>(sh_a[par], sh_b[par], wave);
-    const Affine total = fold_waves<NW>(sh_a[par], sh_b[par], NW);
+    Affine before, total;
+    wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, before, total);
     bool has_entry = false;
     float entry = 0.0f;
     if (has_carry) {
@@ -105,8 +105,8 @@ __global__ __launch_bounds__(64 * NW) void stream_kernel(TileArgs p) {
       sh_b[par][wave] = r.total.b;
     }
     __syncthreads();
-    const Affine before = fold_waves<NW>(sh_a[par], sh_b[par], wave);
-    const Affine total = fold_waves<NW>(sh_a[par], sh_b[par], NW);
+    Affine before, total;
+    wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, before, total);
     bool has_entry = false;
     float entry = 0.0f;
     if (has_carry) {

@@ -62,7 +62,6 @@ __global__ __launch_bounds__(64 * NW) void sweep_kernel(TileArgs p) {
   };
 
   float own_out = 0.0f;  // value that left this walker's previous tile of the current row
-  bool failed = false;   // a bounded wait ran out: what follows in that row is written as NaN
 
   auto finish = [&](long long n, const Item& it, const RowPtrs<T>& q, TileData<S, VEC, MODE> d, bool last) {
     const int t = it.t;
@@ -79,27 +78,24 @@ __global__ __launch_bounds__(64 * NW) void sweep_kernel(TileArgs p) {
       sh_b[par][wave] = r.total.b;
     }
     __syncthreads();
-    const Affine before = fold_waves<NW>(sh_a[par], sh_b[par], wave);
+    Affine before, total;
+    wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, before, total);
     if (wave == 0) {
       uint64_t* desc = p.desc + 2 * (it.row * K);
-      const Affine total = fold_waves<NW>(sh_a[par], sh_b[par], NW);
       if (lane == 0 && t + 1 < K) {
         st_desc(desc + 2 * (long long)t, pack_desc((seq << 2) | STATUS_AGGREGATE, total.a));
         st_desc(desc + 2 * (long long)t + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, total.b));
       }
-      if (t < M) failed = false;  // a new row starts clean
       const int need = t < M - 1 ? t : M - 1;
       float carry_in = 0.0f;
       if (t > 0) {
         Affine acc = {1.0f, 0.0f};
-        if (need > 0 && !failed) {
-          if (!gather_maps(desc, t, need, seq, lane, p.spin_limit, acc)) {
-            failed = true;
-            if (lane == 0) __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-        }
-        if (failed) {
-          carry_in = __builtin_nanf("");
+        bool ok = true;
+        if (need > 0) ok = gather_maps(desc, t, need, seq, lane, p.spin_limit, acc);
+        if (!ok) {
+          // the wait ran out: the value entering the tile from the row's own data instead
+          if (lane == 0) __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          carry_in = recompute_entry<VEC, MODE, DESC>(q, rv, t * TILE_SLOTS, lane);
         } else if (t < M) {
           carry_in = acc.b;  // the maps reach back to the row start
         } else {

@@ -94,7 +94,6 @@ __global__ __launch_bounds__(64 * NW) void team_kernel(TileArgs p) {
   }
 
   float own_out = 0.0f;  // value that left this walker's previous tile
-  bool failed = false;   // a bounded wait ran out: the rest of the row is written as NaN
 
   // Everything after the loads of tile t: scan, exchange inside the workgroup and the team, apply, store.
   auto finish = [&](int t, const TileData<S, VEC, MODE>& d, auto interior_tag, bool last) {
@@ -108,9 +107,9 @@ __global__ __launch_bounds__(64 * NW) void team_kernel(TileArgs p) {
       sh_b[par][wave] = r.total.b;
     }
     __syncthreads();
-    const Affine before = fold_waves<NW>(sh_a[par], sh_b[par], wave);
+    Affine before, total;
+    wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, before, total);
     if (wave == 0) {
-      const Affine total = fold_waves<NW>(sh_a[par], sh_b[par], NW);
       if (lane == 0 && t + 1 < K) {
         st_desc(desc + 2 * (long long)t, pack_desc((seq << 2) | STATUS_AGGREGATE, total.a));
         st_desc(desc + 2 * (long long)t + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, total.b));
@@ -119,9 +118,12 @@ __global__ __launch_bounds__(64 * NW) void team_kernel(TileArgs p) {
       float carry_in = 0.0f;
       if (t > 0) {
         Affine acc = {1.0f, 0.0f};
-        if (need > 0 && !failed) failed = !gather_maps(desc, t, need, seq, lane, p.spin_limit, acc);
-        if (failed) {
-          carry_in = __builtin_nanf("");
+        bool ok = true;
+        if (need > 0) ok = gather_maps(desc, t, need, seq, lane, p.spin_limit, acc);
+        if (!ok) {
+          // the wait ran out: the value entering the tile from the row's own data instead
+          if (lane == 0) __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          carry_in = recompute_entry<VEC, MODE, DESC>(q, rv, t * TILE_SLOTS, lane);
         } else if (t < M) {
           carry_in = acc.b;  // the maps reach back to the row start
         } else {
@@ -174,8 +176,6 @@ __global__ __launch_bounds__(64 * NW) void team_kernel(TileArgs p) {
   }
   for (int i = i_hi; i < n_own; ++i) edge_tile(i);
 
-  if (wave == 0 && failed && lane == 0)
-    __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (n_own == 0 && threadIdx.x == 0) leaf_count = signal_tile_done_begin(p, wg);
   if (threadIdx.x == 0) signal_tile_done_end(p, wg, seq, leaf_count);
 }

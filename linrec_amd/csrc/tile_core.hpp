@@ -318,15 +318,65 @@ __device__ __forceinline__ void tile_apply_store(const TileData<S, VEC, MODE>& d
   }
 }
 
-// Composition of the aggregates of waves 0 .. count-1 held in LDS.
-template <int NW>
-__device__ __forceinline__ Affine fold_waves(const float* sh_a, const float* sh_b, int count) {
-  Affine acc = {1.0f, 0.0f};
-#pragma unroll
-  for (int w = 0; w < NW; ++w) {
-    if (w < count) acc = w == 0 ? Affine{sh_a[0], sh_b[0]} : compose(acc, {sh_a[w], sh_b[w]});
+// The value carried into scan-order slot `u_end` of a row (slots of VEC elements), computed by one wave
+// from the row's own data.  The slow way out for a wave whose bounded wait for other workgroups'
+// results ran out: correct whatever the others are doing (or not doing), so that a kernel whose
+// workgroups wait for each other never has to hand out a wrong value.  It walks the row one element per
+// lane and step (64 elements a step): as slow as it gets, and light on registers, which matters because
+// it is compiled into kernels whose every register is spoken for.
+template <int VEC, int MODE, bool DESC, typename T>
+__device__ __forceinline__ float recompute_entry(const RowPtrs<T> q, const RowView rv, int u_end, int lane) {
+  // the elements in front of slot u_end, as a row of its own in one-element slots
+  RowView part;
+  if constexpr (DESC) {
+    const int first = (rv.nslots - u_end) * VEC;  // lowest virtual index that takes part
+    part.lo = first < rv.lo ? rv.lo : first;
+    part.hi = rv.hi;
+  } else {
+    const int end = u_end * VEC;  // one past the highest virtual index that takes part
+    part.lo = rv.lo;
+    part.hi = end > rv.hi ? rv.hi : end;
   }
-  return acc;
+  part.nslots = part.hi;
+  const int count = part.hi - part.lo;
+  float carry = 0.0f;
+  bool has = false;
+  for (int e = 0; e < count; e += 64) {
+    // scan-order slot of element e: ascending, virtual index lo + e; descending, hi - 1 - e
+    const int u = DESC ? e : part.lo + e;
+    TileData<1, 1, MODE> d;
+    tile_load<1, 1, MODE, DESC, false>(d, q, part, u, lane, false);
+    if constexpr (MODE == MODE_FWD) {
+      if (e == 0 && lane == 0) d.cs[0][0] = 0.0f;  // the row's first coefficient takes no part
+    }
+    TileScan<1, 1> r;
+    tile_scan<1, 1, MODE>(d, r);
+    carry = has ? fmaf(carry, r.total.a, r.total.b) : r.total.b;
+    has = true;
+  }
+  return carry;
+}
+
+// The maps of the NW <= 16 waves of a workgroup lie in LDS.  Every wave folds them for itself by a
+// four-step scan over the lanes of one DPP row (lane w: wave w's map, identity elsewhere) and takes what
+// it needs out of it with v_readlane, so both results are wave-uniform scalars: the composition of the
+// waves in front of `wave` (the identity for wave 0) and of all NW waves.
+template <int NW>
+__device__ __forceinline__ void wave_prefixes(const float* sh_a, const float* sh_b, int wave, int lane, Affine& before,
+                                              Affine& total) {
+  static_assert(NW <= 16, "one DPP row holds the waves' maps");
+  float a[1] = {1.0f}, b[1] = {0.0f};
+  if (lane < NW) {
+    a[0] = sh_a[lane];
+    b[0] = sh_b[lane];
+  }
+  if constexpr (NW > 1) scan_step<DPP_ROW_SHR1, 0xf>(a, b);
+  if constexpr (NW > 2) scan_step<DPP_ROW_SHR2, 0xf>(a, b);
+  if constexpr (NW > 4) scan_step<DPP_ROW_SHR4, 0xf>(a, b);
+  if constexpr (NW > 8) scan_step<DPP_ROW_SHR8, 0xf>(a, b);
+  total = {read_lane(a[0], NW - 1), read_lane(b[0], NW - 1)};
+  // lane w-1 holds waves 0 .. w-1; for wave 0 this reads lane 63, which still holds the identity
+  before = {read_lane(a[0], (wave - 1) & 63), read_lane(b[0], (wave - 1) & 63)};
 }
 
 }  // namespace linrec

@@ -24,7 +24,7 @@ namespace linrec {
 // descriptor words per tile.  Everything but `seq` and `gave_up` is zero between launches.
 struct alignas(16) CarryHeader {
   uint32_t seq;      // launch sequence number; descriptor flags of other launches never match
-  uint32_t gave_up;  // number of look-backs that hit the poll limit (results are then invalid)
+  uint32_t gave_up;  // waits that hit the poll limit (the value was then computed from the row's own data)
   uint32_t pad[2];
 };
 constexpr uint32_t SEQ_MASK = 0x3fffffffu;
@@ -69,11 +69,12 @@ __device__ __forceinline__ void st_desc(uint64_t* p, uint64_t v) {
 // (k >= 1).  `desc` points at the row's first descriptor.  Each 64-bit word carries its own flag,
 // so a reader never needs a fence: a word is either from this launch (flag matches) or ignored.
 //
-// The wait is bounded: after `spin_limit` fruitless polls the tile records the failure in the
-// header and carries NaN, so a protocol error or a foreign writer ends in wrong, flagged results
-// rather than in a wave that never exits.
+// The wait is bounded: after `spin_limit` fruitless polls the tile counts the event in the header and
+// reports it (`ok` = false); the caller then computes the value from the row's own data
+// (recompute_entry), so neither a wave that never exits nor a wrong result can come of it.
 __device__ __forceinline__ float look_back(const uint64_t* desc, int k, uint32_t seq, int lane,
-                                           int spin_limit, CarryHeader* hdr) {
+                                           int spin_limit, CarryHeader* hdr, bool& ok) {
+  ok = true;
   Affine acc = {1.0f, 0.0f};  // composition of the tiles already folded (nearest ones)
   int pred = k - 1;           // lane 0 inspects `pred`, lane i inspects pred - i
   int polls = 0;
@@ -104,7 +105,8 @@ __device__ __forceinline__ float look_back(const uint64_t* desc, int k, uint32_t
     if (wait_mask & below) {
       if (++polls > spin_limit) {
         if (lane == 0) __hip_atomic_fetch_add(&hdr->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return __builtin_nanf("");
+        ok = false;
+        return 0.0f;
       }
       __builtin_amdgcn_s_sleep(1);
       continue;  // a needed predecessor has not published yet: poll the same window again
@@ -219,12 +221,12 @@ __global__ __launch_bounds__(64 * NW) void tile_kernel(TileArgs p) {
     }
     __syncthreads();
     LINREC_STAMP(2);
-    const Affine before = fold_waves<NW>(sh_a, sh_b, wave);  // the waves in front of this one
+    Affine before, total;  // the waves in front of this one, and all of them
+    wave_prefixes<NW>(sh_a, sh_b, wave, lane, before, total);
     float tile_in = 0.0f;
     if constexpr (CARRY) {
       uint64_t* desc = p.desc + 2 * (row * p.tiles_per_row);
       if (wave == 0) {
-        const Affine total = fold_waves<NW>(sh_a, sh_b, NW);
         float carry_in = 0.0f;
         if (k == 0) {
           if (lane == 0) st_desc(desc + 1, pack_desc((seq << 2) | STATUS_INCLUSIVE, total.b));
@@ -234,7 +236,9 @@ __global__ __launch_bounds__(64 * NW) void tile_kernel(TileArgs p) {
             st_desc(desc + 2 * k + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, total.b));
           }
           LINREC_STAMP(3);
-          carry_in = look_back(desc, k, seq, lane, p.spin_limit, p.ws);
+          bool ok;
+          carry_in = look_back(desc, k, seq, lane, p.spin_limit, p.ws, ok);
+          if (!ok) carry_in = recompute_entry<VEC, MODE, DESC>(q, rv, k * TILE_SLOTS, lane);
           LINREC_STAMP(4);
           if (lane == 0)
             st_desc(desc + 2 * k + 1,

@@ -130,21 +130,25 @@ def running_error_scale(x, c, reverse=False):
                reverse=reverse, dtype=np.float64)
 
 
-def error_report(got, want64, scale=None):
+def error_report(got, want64, scale=None, mixed_rtol=1e-5, mixed_atol=1e-5):
     """Error figures used by the parity tests; `got` fp32, `want64` float64 ground truth.
 
     normwise  = max|got - want| / max|want|          (headline bar: <= 1e-5)
+    mixed     = share of elements with |got - want| <= rtol * |want| + atol * rms(want), rtol = atol = 1e-5
+                (an elementwise bar: small values next to large ones cannot hide behind max|want|)
     maxabs    = max|got - want|                      (the reference's own figure, eval/test.py:24)
     reassoc   = max(|got - want| / (2^-24 * scale))  (in units of fp32 roundoff of the running bound)
     """
     got = np.asarray(got, dtype=np.float64)
     want64 = np.asarray(want64, dtype=np.float64)
     if got.size == 0:
-        return {"normwise": 0.0, "maxabs": 0.0, "reassoc": 0.0}
+        return {"normwise": 0.0, "maxabs": 0.0, "reassoc": 0.0, "mixed": 1.0}
     diff = np.abs(got - want64)
     denom = np.max(np.abs(want64))
+    rms = float(np.sqrt(np.mean(want64 * want64)))
     rep = {"maxabs": float(diff.max()),
-           "normwise": float(diff.max() / denom) if denom > 0 else float(diff.max())}
+           "normwise": float(diff.max() / denom) if denom > 0 else float(diff.max()),
+           "mixed": float(np.mean(diff <= mixed_rtol * np.abs(want64) + mixed_atol * rms))}
     if scale is not None:
         s = np.asarray(scale, dtype=np.float64)
         ok = s > 0

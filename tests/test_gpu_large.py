@@ -20,7 +20,7 @@ CASES = {
     "column_f32": (4194304, 520, True, False, torch.float32, "COLUMN"),
     "segment_f32": (4000, 537000, True, True, torch.float32, "SEGMENT"),
     "colblock_f32": (16000, 134300, True, True, torch.float32, "COLUMN"),
-    "sweep_f32": (20, 1 << 27, False, True, torch.float32, "SWEEP"),
+    "drift_f32": (20, 1 << 27, False, True, torch.float32, "DRIFT"),  # (its backward: teams that wait, SWEEP)
     "team_f32": (18, (1 << 27) + 12, False, False, torch.float32, "TEAM"),
     "stream_bf16": (70000, 32768, False, True, torch.bfloat16, "STREAM"),
 }

@@ -54,12 +54,13 @@ def test_planner_follows_the_compute_unit_count():
             assert lib.linrec_compute_units() == cus
             for is_bwd in (False, True):
                 p = nat.plan(x, False, is_bwd)
-                if cus == 20:  # 16 rows are "many" for 20 CUs: one workgroup per row, nobody waits
+                if cus == 20 and is_bwd:  # 16 rows are "many" for 20 CUs: one workgroup per row, nobody waits
                     assert p["family"] == nat.FAMILY_STREAM and p["workspace_bytes"] == 0
                     continue
-                assert p["family"] == nat.FAMILY_SWEEP
-                # forward: at most two workgroups per CU, backward one; whole teams only
-                assert p["grid"] <= (1 if is_bwd else 2) * cus and p["grid"] % p["tasks"] == 0
+                # forward: teams whose tiles are stored two steps late; backward: teams that wait (tiles of 16384)
+                assert p["family"] == (nat.FAMILY_SWEEP if is_bwd else nat.FAMILY_DRIFT)
+                # one workgroup per CU at most; whole teams only
+                assert p["grid"] <= cus and p["grid"] % p["tasks"] == 0
                 seen[(cus, is_bwd)] = p["grid"]
             # one team of workgroups per row: never more workgroups than CUs
             t = nat.plan(torch.empty(8, 1048580), False, False)
@@ -67,7 +68,7 @@ def test_planner_follows_the_compute_unit_count():
             # one workgroup per row from half the CUs on, teams below
             assert nat.plan(torch.empty(cus // 2 + 1, 65540))["family"] == nat.FAMILY_STREAM
             assert nat.plan(torch.empty(cus // 2, 65540))["family"] == nat.FAMILY_TEAM
-        assert seen[(256, False)] == 256 and seen[(128, False)] == 256 and seen[(64, False)] == 128
+        assert seen[(256, False)] == 256 and seen[(128, False)] == 128 and seen[(64, False)] == 64
         assert seen[(256, True)] == 256 and seen[(128, True)] == 128 and seen[(64, True)] == 64
         # a team that cannot be resident at once is refused rather than left to wait for absent mates
         lib.linrec_set_compute_units(8)
@@ -107,13 +108,17 @@ class TestPlanner:
         names = nat.kernel_table()
         p1 = _plan((64, 4096))
         assert p1["family"] == nat.FAMILY_TILE and p1["carry"] == 0 and p1["grid"] == 64
-        p2 = _plan((512, 65536))
-        assert p2["family"] == nat.FAMILY_STREAM and p2["grid"] == 512 and p2["workspace_bytes"] == 0
+        p2 = _plan((512, 65536))  # teams of 8 workgroups per row of 8 tiles, 32 teams, a tile stored two steps late
+        assert p2["family"] == nat.FAMILY_DRIFT and (p2["slots"], p2["tasks"], p2["grid"], p2["tiles_per_row"]) == (4, 8, 256, 8)
+        assert "drift_w8_s4_MODE_FWD_0" == names[p2["kernel_id"]] and p2["workspace_bytes"] > 0
+        p2b = _plan((512, 65536), is_bwd=True)  # the backward holds three tensors: tiles of 4096 elements
+        assert p2b["family"] == nat.FAMILY_DRIFT and (p2b["slots"], p2b["tasks"], p2b["grid"], p2b["tiles_per_row"]) == (2, 16, 256, 16)
+        assert "drift_w8_s2_MODE_BWD_1" == names[p2b["kernel_id"]]
         p3 = _plan((16384, 2048), reverse=True)
         assert (p3["waves"], p3["slots"], p3["carry"]) == (4, 2, 0) and "FWD_1" in names[p3["kernel_id"]]
-        p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 16 that could go on to further rows
-        assert p4["family"] == nat.FAMILY_SWEEP and p4["carry"] == 1 and p4["workspace_bytes"] > 0
-        assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (16, 256, 128)
+        p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 64 (half a row in flight each) that go from row to row
+        assert p4["family"] == nat.FAMILY_DRIFT and p4["carry"] == 1 and p4["workspace_bytes"] > 0
+        assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (64, 256, 128)
         p4bw = _plan((16, 1048576), is_bwd=True)  # the backward takes tiles of 16384 elements
         assert (p4bw["family"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_SWEEP, 8, 16, 256, 64)
         p4r = _plan((16, 1048576 + 4))  # a ragged last tile: one team per row
@@ -164,33 +169,35 @@ class TestPlanner:
         p = _plan((300, 20000), tuning=nat.Tuning(nat.FAMILY_STREAM, 16, 2))
         assert p["family"] == nat.FAMILY_STREAM and p["block"] == 1024
 
-    def test_sweep_is_chosen_where_rows_do_not_spread_evenly_otherwise(self):
+    def test_teams_are_chosen_where_rows_are_whole_tiles(self):
         fam = lambda shape, bwd=False, **kw: nat.plan(torch.empty(shape, **kw), False, bwd)["family"]
-        assert fam((300, 65536)) == nat.FAMILY_SWEEP and fam((96, 65536)) == nat.FAMILY_SWEEP
-        assert fam((256, 65536)) == nat.FAMILY_STREAM and fam((200, 65536)) == nat.FAMILY_STREAM
-        # multiples of 256 rows: the forward is stream's; the backward sweeps from 512 rows on, except
-        # rows of 16 tiles and more beyond 1024 rows
-        assert fam((512, 65536)) == nat.FAMILY_STREAM and fam((512, 65536), True) == nat.FAMILY_SWEEP
-        assert fam((1024, 131072)) == nat.FAMILY_STREAM and fam((1024, 131072), True) == nat.FAMILY_SWEEP
-        assert fam((4096, 65536), True) == nat.FAMILY_SWEEP and fam((1536, 131072), True) == nat.FAMILY_STREAM
-        assert fam((256, 65536), True) == nat.FAMILY_STREAM
+        D, W, ST = nat.FAMILY_DRIFT, nat.FAMILY_SWEEP, nat.FAMILY_STREAM
+        # fp32 rows of whole tiles, up to 2048 of them: the forward always, the backward from 128 rows on and
+        # for rows up to 131072 elements
+        for shape in [(300, 65536), (96, 65536), (256, 65536), (200, 65536), (512, 65536), (1024, 131072), (2048, 65536),
+                      (16, 1 << 20), (8, 1 << 22), (4, 1 << 20)]:
+            assert fam(shape) == D, shape
+        for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 16384)]:
+            assert fam(shape, True) == D, shape
+        assert fam((96, 65536), True) == W and fam((16, 1 << 20), True) == W and fam((512, 262144), True) == W
+        # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
+        assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
+        assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # teams of at most 64 would leave most of the chip idle
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
-        # stream tiles of 16384 elements: one workgroup per CU at most, or long rows, of whole such tiles
-        assert slots((512, 65536)) == 4 and slots((256, 32768)) == 8 and slots((512, 131072)) == 8
-        assert slots((256, 32768 + 8192)) == 4 and slots((2048, 131072), True) == 8
-        assert slots((1024, 65536)) == 8
+        # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
+        assert slots((4096, 65536)) == 8 and slots((2304, 131072), True) == 8
+        assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
-        assert slots((1365, 24576)) == 4 and slots((838, 40000)) == 4 and slots((800, 36000)) == 2
-        assert fam((2048, 131072), True) == nat.FAMILY_STREAM     # the backward sweep rule ends at 1024 rows
+        assert slots((4000, 24576)) == 4 and slots((838, 40000)) == 4 and slots((800, 36000)) == 2
         assert fam((300, 65536 + 4)) == nat.FAMILY_STREAM          # ragged last tile
         # ... whose rows beyond one per CU, if few, go to a second launch of their own (teams per row)
         p = nat.plan(torch.empty(300, 65536 + 4))
         assert (p["tail_rows"], p["grid"]) == (44, 256) and p["workspace_bytes"] > 0
         assert [nat.plan(torch.empty(n, 65536 + 4))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
         assert nat.plan(torch.empty(300, 65536 + 4), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
-        assert fam((300, 16384)) == nat.FAMILY_STREAM              # two tiles per row: not worth an exchange
-        assert fam((8, 1 << 20)) == nat.FAMILY_TEAM                # fewer than 16 rows
+        assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
+        assert fam((8, (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
         assert fam((300, 65536), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
         assert fam((16, 1 << 20), dtype=torch.bfloat16) == nat.FAMILY_TEAM
         # 16-bit backward: one team per row where teams of 256 / rows workgroups fill the chip
@@ -199,11 +206,13 @@ class TestPlanner:
         assert [hb(n) for n in (96, 100, 160)] == [nat.FAMILY_SWEEP] * 3
         assert fam((64, 262144), dtype=torch.float16) == nat.FAMILY_SWEEP and fam((64, 262144), True) == nat.FAMILY_SWEEP
         pf, pb = nat.plan(torch.empty(300, 65536)), nat.plan(torch.empty(300, 65536), False, True)
-        assert (pf["tasks"], pf["grid"]) == (8, 512) and (pb["tasks"], pb["grid"]) == (8, 256)
-        p = nat.plan(torch.empty(40, 8192 * 24))                    # 24 tiles: teams of 12
+        assert (pf["tasks"], pf["grid"]) == (8, 256) and (pb["tasks"], pb["grid"]) == (16, 256)
+        p = nat.plan(torch.empty(40, 8192 * 24))                    # 24 tiles: teams of 24, 10 of them
         p2 = nat.plan(torch.empty(300, 4096 * 9))                   # whole tiles of 4096 elements only
-        assert (p2["family"], p2["slots"], p2["tasks"], p2["tiles_per_row"]) == (nat.FAMILY_SWEEP, 2, 9, 9)
-        assert p["family"] == nat.FAMILY_SWEEP and p["tasks"] == 12
+        assert (p2["family"], p2["slots"], p2["tasks"], p2["tiles_per_row"], p2["grid"]) == (D, 2, 9, 9, 252)
+        assert p["family"] == D and (p["tasks"], p["grid"]) == (24, 240)
+        p = nat.plan(torch.empty(40, 8192 * 24), False, True)       # the backward of fewer than 128 rows waits
+        assert p["family"] == W and p["tasks"] == 12
 
     def test_few_rows_on_a_strided_scan_axis_are_cut_into_segments(self):
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
@@ -344,7 +353,7 @@ class TestPlanner:
         assert lib.linrec_plan_f32(None, 4, 10, 5, 1, 0, 0, None, ctypes.byref(plan)) == -1  # rows overlap
         assert lib.linrec_plan_f32(None, 4, 2 ** 31, 2 ** 31, 1, 0, 0, None, ctypes.byref(plan)) == -4
         assert lib.linrec_workspace_bytes(16, 1 << 20, 1 << 20, 1, 0, 0, None) > 0
-        assert lib.linrec_workspace_bytes(512, 65536, 65536, 1, 0, 0, None) == 0
+        assert lib.linrec_workspace_bytes(4096, 65536, 65536, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
         assert lib.linrec_workspace_bytes_for_tiles(0) == 0
         assert lib.linrec_workspace_bytes_for_tiles(1000) >= 16 + 16 * 1000
 

@@ -40,10 +40,20 @@ def truth(x, c, dy, reverse):
     return y, dx, dc
 
 
-def check_close(got, want64, what, tol=TOL_NORMWISE):
+TOL_MIXED_SHARE = 0.999  # share of elements within |d| <= 1e-5 |t| + 1e-5 rms(t) of the float64 recurrence
+
+
+def check_close(got, want64, what, tol=TOL_NORMWISE, mixed_share=TOL_MIXED_SHARE):
+    """The parity bar: the normwise figure (max|got - truth| / max|truth| <= tol), and next to it the
+    elementwise mixed tolerance |d| <= 1e-5 |t| + 1e-5 rms(t), which all but a sliver of the elements
+    must meet (a reassociated fp32 scan is a few roundoffs of the running bound off, which can exceed
+    1e-5 of an element that happens to be tiny).  16-bit storage is held to the normwise bar alone:
+    its rounding unit is far above 1e-5."""
     got = got.detach().double().cpu().numpy()
     assert got.shape == want64.shape, (what, got.shape, want64.shape)
     assert np.isfinite(got).all(), f"{what}: non-finite values in the result"
     rep = oracle.error_report(got, want64)
     assert rep["normwise"] <= tol, f"{what}: {rep}"
+    if tol <= TOL_NORMWISE:
+        assert rep["mixed"] >= mixed_share, f"{what}: {rep}"
     return rep
