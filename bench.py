@@ -13,8 +13,8 @@ Prints ONE JSON line.  `value` is the achieved bandwidth of the step in algorith
 d_outputs, coeffs, outputs, write d_inputs, d_coeffs), i.e. 32 * elements / time per step.
 `roofline` prices the dominant kernel (backward) against the 8 TB/s HBM peak with its duration
 measured by HIP events on the launch stream; `roofline_fwd` does the same for the forward kernel.
-`cpu_baseline` times the CPU checker's restatement of the reference's per-timestep host loop on
-this box's cores (a reported baseline, not a target).
+`cpu_baseline` times the CPU checker's restatement of the reference's eager-torch host loop on this
+box's cores, with a numpy and a multi-threaded C line beside it (reported baselines, not targets).
 """
 import argparse
 import json
@@ -33,11 +33,14 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("C1", "tile_w8_s2_v4_MODE_FWD_0_0"): 3.195e6,
     ("C1", "tile_w8_s2_v4_MODE_BWD_1_0"): 5.362e6,
+    ("C2", "drift_w8_s4_MODE_FWD_0"): 403.73e6,
+    ("C2", "drift_w8_s2_MODE_BWD_1"): 674.56e6,
     ("C2", "stream_w8_s4_MODE_FWD_0"): 402.71e6,
     ("C2", "stream_w8_s4_MODE_BWD_1"): 671.42e6,
     ("C2", "sweep_w8_s4_MODE_BWD_1"): 673.19e6,
     ("C3", "tile_w4_s2_v4_MODE_FWD_1_0"): 402.58e6,
     ("C3", "tile_w4_s2_v4_MODE_BWD_0_0"): 676.67e6,
+    ("C4", "drift_w8_s4_MODE_FWD_0"): 202.22e6,
     ("C4", "sweep_w8_s4_MODE_FWD_0"): 202.13e6,
     ("C4", "sweep_w8_s8_MODE_BWD_1"): 336.73e6,
     ("C5", "column_v2_u8_MODE_FWD_0"): 805.12e6,
@@ -114,40 +117,51 @@ def event_series_ms(torch, fn, iters):
     return sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(iters))
 
 
-def cpu_baseline(cfg, host, budget_s=25.0):
-    """The checker's numpy restatement of the reference's host path (one vector operation per
-    timestep over all rows, linrec/impl/python/ops.py:16-18 and :32-40) on a bounded sample of the
-    same workload, plus the plain C loop as a second line."""
+def cpu_baseline(cfg, host, budget_s=20.0):
+    """The reference's host path on this box's cores, restated by the CPU checker and timed on a bounded
+    sample of the same workload (a reported baseline, not a target): the eager-torch loop as the
+    reference writes it (one multiply-add over all rows per timestep, linrec/impl/python/ops.py:16-18
+    and :32-40), with torch's thread count; the same loop in numpy; and a plain C loop per row with the
+    rows spread over OpenMP threads."""
     import numpy as np
+    import torch
     from oracle import oracle
-    x, c, dy = (t.numpy() for t in host)
-    n, L = x.shape
-    rows = n
-    # bound the sample: one probe on a few rows, then scale the row count to the time budget
+    xt, ct, dyt = host
+    n, L = xt.shape
+    # bound the sample: one probe of a few hundred timesteps, then as many timesteps as fit the budget
+    probe = min(L, 512)
     t0 = time.perf_counter()
-    probe = min(n, 8)
-    oracle.fwd_numpy(x[:probe], c[:probe], cfg["reverse"], dtype=np.float32)
-    per_pass = time.perf_counter() - t0  # dominated by the per-timestep overhead, nearly row-independent
-    if per_pass * 2.5 > budget_s:
-        L_s = max(1, int(L * budget_s / (per_pass * 2.5)))
-    else:
-        L_s = L
-    xs, cs, dys = x[:rows, :L_s], c[:rows, :L_s], dy[:rows, :L_s]
-    t0 = time.perf_counter()
-    y = oracle.fwd_numpy(xs, cs, cfg["reverse"], dtype=np.float32)
-    oracle.bwd_numpy(dys, cs, y, cfg["reverse"], dtype=np.float32)
-    t_np = time.perf_counter() - t0
-    elems = rows * L_s
-    t0 = time.perf_counter()
-    y = oracle.fwd(xs, cs, cfg["reverse"], dtype=np.float32)
-    oracle.bwd(dys, cs, y, cfg["reverse"], dtype=np.float32)
-    t_c = time.perf_counter() - t0
+    oracle.fwd_torch(xt[:, :probe], ct[:, :probe], cfg["reverse"])
+    per_step = (time.perf_counter() - t0) / probe
+    L_s = L if per_step * L * 2.6 <= budget_s else max(1, int(budget_s / (per_step * 2.6)))
+    xs, cs, dys = xt[:, :L_s], ct[:, :L_s], dyt[:, :L_s]
+    elems = n * L_s
     gb = (FWD_BYTES_PER_ELEM + BWD_BYTES_PER_ELEM) * elems / 1e9
-    return ({"value": gb / t_np, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"fwd+bwd of rows[:{rows}], timesteps[:{L_s}] of the same inputs, per-timestep numpy loop, "
-                       f"{t_np:.2f} s, host has {os.cpu_count()} cpus"},
-            {"value": gb / t_c, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"same sample, sequential C loop per row (includes dense copies made by the wrapper), {t_c:.2f} s"})
+    sample = f"fwd+bwd of all {n} rows, timesteps[:{L_s}] of the same inputs"
+
+    t0 = time.perf_counter()
+    y = oracle.fwd_torch(xs, cs, cfg["reverse"])
+    oracle.bwd_torch(dys, cs, y, cfg["reverse"])
+    t_torch = time.perf_counter() - t0
+    xn, cn, dyn = (t.numpy() for t in (xs, cs, dys))
+    t0 = time.perf_counter()
+    yn = oracle.fwd_numpy(xn, cn, cfg["reverse"], dtype=np.float32)
+    oracle.bwd_numpy(dyn, cn, yn, cfg["reverse"], dtype=np.float32)
+    t_np = time.perf_counter() - t0
+    threads = oracle.threads()
+    t0 = time.perf_counter()
+    yc = oracle.fwd(xn, cn, cfg["reverse"], dtype=np.float32)
+    oracle.bwd(dyn, cn, yc, cfg["reverse"], dtype=np.float32)
+    t_c = time.perf_counter() - t0
+    cpus = os.cpu_count()
+    return ({"value": gb / t_torch, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+             "sample": f"{sample}, eager-torch loop over timesteps (the reference's host path), {t_torch:.2f} s, "
+                       f"torch.get_num_threads() = {torch.get_num_threads()}, host has {cpus} cpus"},
+            {"value": gb / t_np, "unit": "GB/s", "cores": 1, "kind": "port",
+             "sample": f"same sample, the same loop in numpy, {t_np:.2f} s"},
+            {"value": gb / t_c, "unit": "GB/s", "cores": threads, "kind": "port",
+             "sample": f"same sample, sequential C loop per row, rows over {threads} OpenMP threads "
+                       f"(includes dense copies made by the wrapper), {t_c:.2f} s"})
 
 
 def main():
@@ -298,9 +312,9 @@ def main():
         "device": torch.cuda.get_device_name(0),
     }
     if not a.no_cpu and a.dtype == "f32":
-        np_line, c_line = cpu_baseline(cfg, host0)
-        out["cpu_baseline"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in np_line.items()}
-        out["cpu_baseline_c_loop"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c_line.items()}
+        lines = cpu_baseline(cfg, host0)
+        for key, line in zip(("cpu_baseline", "cpu_baseline_numpy", "cpu_baseline_c_loop"), lines):
+            out[key] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in line.items()}
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

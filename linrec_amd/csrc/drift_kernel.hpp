@@ -208,22 +208,23 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     if constexpr (MODE == MODE_BWD) now.d = d;
     now.it = it;
   };
-  // The last tile lies in P[A] and the one before it in P[(A + 2) % 3]: nothing left to overlap with.
+  // The last tile lies in P[A] and the one before it in P[(A + 2) % 3]: nothing left to overlap with, so
+  // both are asked for at once, and one barrier serves both.
   auto finish = [&]<int A>(std::integral_constant<int, A>) {
     constexpr int PREV = (A + 2) % 3;
-    if (items >= 2) {
-      if (wave == 0) {
-        const float cin = resolve(P[PREV], 0, 0);
+    if (wave == 0) {
+      uint64_t w0 = 0, w1 = 0, v0 = 0, v1 = 0;
+      if (items >= 2) ask(P[PREV].it, w0, w1);
+      ask(P[A].it, v0, v1);  // (published moments ago: if the words are not there yet, resolve polls for them)
+      if (items >= 2) {
+        const float cin = resolve(P[PREV], w0, w1);
         if (lane == 0) sh_carry[2] = cin;
       }
-      __syncthreads();
-      store_pending(P[PREV], sh_carry[2]);
-    }
-    if (wave == 0) {
-      const float cin = resolve(P[A], 0, 0);
+      const float cin = resolve(P[A], v0, v1);
       if (lane == 0) sh_carry[3] = cin;
     }
     __syncthreads();
+    if (items >= 2) store_pending(P[PREV], sh_carry[2]);
     store_pending(P[A], sh_carry[3]);
   };
   using I0 = std::integral_constant<int, 0>;

@@ -18,12 +18,20 @@
  * O(L^2) explicit-sum formulation differentiated by autograd plus central finite
  * differences.  Every function below is covered by at least one of those.
  *
+ * Rows run in parallel (OpenMP); each row is the plain sequential loop.
+ *
  * Layout: element (r, l) of a tensor lives at base[r*row_stride + l*elem_stride]
  * (strides in elements), so dense rows, padded rows and transposed views are all
  * addressed the same way.
  */
+#include <omp.h>
 #include <stddef.h>
 #include <stdint.h>
+
+/* Rows are independent (linrec/impl/cuda/linrec_pipe.cuh:14): the loops below run them on
+ * several threads.  The timed CPU baseline states how many; everything else leaves OpenMP's default. */
+int oracle_max_threads(void) { return omp_get_max_threads(); }
+void oracle_set_threads(int n) { if (n > 0) omp_set_num_threads(n); }
 
 #define DEFINE_ORACLE(T, SUFFIX)                                                              \
   /* forward: linrec_ref.cuh:63-68 (explicit first element), ops.py:16-18 */                  \
@@ -31,6 +39,7 @@
                                   int64_t seqlen, int64_t row_stride, int64_t elem_stride,    \
                                   int reverse) {                                              \
     if (seqlen <= 0) return;                                                                  \
+    _Pragma("omp parallel for schedule(static)")                                              \
     for (int64_t r = 0; r < numseq; ++r) {                                                    \
       const T* xr = x + r * row_stride;                                                       \
       const T* cr = c + r * row_stride;                                                       \
@@ -51,6 +60,7 @@
                                   int64_t numseq, int64_t seqlen, int64_t row_stride,         \
                                   int64_t elem_stride, int reverse) {                         \
     if (seqlen <= 0) return;                                                                  \
+    _Pragma("omp parallel for schedule(static)")                                              \
     for (int64_t r = 0; r < numseq; ++r) {                                                    \
       const T* dyr = dy + r * row_stride;                                                     \
       const T* cr = c + r * row_stride;                                                       \

@@ -39,8 +39,18 @@ def _load():
             getattr(lib, f"oracle_linrec_fwd_{sfx}").restype = None
             getattr(lib, f"oracle_linrec_bwd_{sfx}").argtypes = [p, p, p, p, p, i64, i64, i64, i64, i]
             getattr(lib, f"oracle_linrec_bwd_{sfx}").restype = None
+        lib.oracle_max_threads.restype = i
+        lib.oracle_set_threads.argtypes = [i]
         _lib = lib
     return _lib
+
+
+def threads(n=None):
+    """Threads the C loops run rows on (OpenMP); `n` sets it.  Returns the number in force."""
+    lib = _load()
+    if n is not None:
+        lib.oracle_set_threads(int(n))
+    return int(lib.oracle_max_threads())
 
 
 def _canon(*arrays, dtype):
@@ -121,6 +131,35 @@ def bwd_numpy(dy, c, y, reverse=False, dtype=np.float64):
     dx = fwd_numpy(dy, cs, reverse=not reverse, dtype=dtype)
     dc = dx * shift_numpy(y, 1 if not reverse else -1, 0.0)
     return dx, dc
+
+
+def fwd_torch(x, c, reverse=False):
+    """The reference's host path as it is written, in eager torch: one multiply-add over all rows per
+    timestep and a column store (linrec/impl/python/ops.py:8-20).  `x`, `c`: CPU torch tensors."""
+    import torch
+    y = torch.empty_like(x)
+    prev = torch.zeros_like(x[..., 0])
+    order = range(x.shape[-1])
+    for i in (reversed(order) if reverse else order):
+        prev = prev * c[..., i] + x[..., i]
+        y[..., i] = prev
+    return y
+
+
+def bwd_torch(dy, c, y, reverse=False):
+    """shift, opposite-direction loop, multiply, in eager torch (linrec/impl/python/ops.py:22-40)."""
+    import torch
+
+    def shift(a, k):  # roll without wrap-around, fill 0
+        out = torch.zeros_like(a)
+        if k > 0:
+            out[..., k:] = a[..., :-k]
+        elif k < 0:
+            out[..., :k] = a[..., -k:]
+        return out
+
+    dx = fwd_torch(dy, shift(c, -1 if not reverse else 1), reverse=not reverse)
+    return dx, dx * shift(y, 1 if not reverse else -1)
 
 
 def running_error_scale(x, c, reverse=False):

@@ -80,6 +80,28 @@ def test_planner_follows_the_compute_unit_count():
         lib.linrec_set_compute_units(0)
 
 
+def test_every_benchmarked_kernel_has_a_measured_traffic_figure():
+    """bench.py reports the HBM bytes per launch that the counters showed for the kernel it times; a
+    planner change that picks another kernel for one of its configurations must not turn that into null
+    unnoticed.  The plan needs no device (256 compute units are assumed without one)."""
+    import bench
+    names = nat.kernel_table()
+    missing = []
+    for key, cfg in bench.CONFIGS.items():
+        shape = cfg["shape"]
+        x = torch.empty(shape[::-1]).t() if cfg["transposed"] else torch.empty(shape)
+        for is_bwd in (False, True):
+            kernel = names[nat.plan(x, cfg["reverse"], is_bwd)["kernel_id"]]
+            if not bench.MEASURED_TRAFFIC_BYTES.get((key, kernel)):
+                missing.append((key, "bwd" if is_bwd else "fwd", kernel))
+    assert not missing, missing
+    for (key, kernel), nbytes in bench.MEASURED_TRAFFIC_BYTES.items():
+        elems = int(np.prod(bench.CONFIGS[key]["shape"])) * (2 if kernel.startswith(("bf16_", "f16_")) else 4)
+        per_elem = 5 if "BWD" in kernel else 3
+        # nothing reads or writes less than the algorithm has to; the segmented scan reads its inputs twice
+        assert 0.97 * per_elem * elems <= nbytes <= 1.75 * per_elem * elems, (key, kernel, nbytes)
+
+
 def test_noalloc_entry_point_rejects_what_its_static_scratch_cannot_hold():
     """linrec_fwd_noalloc turns a call down, before anything touches a device, when the launch would need
     more workspace than the library's static array (no pointer is dereferenced on the host)."""

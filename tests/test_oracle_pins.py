@@ -19,7 +19,20 @@ import torch
 from oracle import oracle
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")
-IMPLS = [("c", oracle.fwd, oracle.bwd), ("numpy", oracle.fwd_numpy, oracle.bwd_numpy)]
+
+
+def _fwd_torch(x, c, reverse=False, dtype=np.float64):
+    t = [torch.from_numpy(np.ascontiguousarray(a, dtype=dtype)) for a in (x, c)]
+    return oracle.fwd_torch(*t, reverse=reverse).numpy()
+
+
+def _bwd_torch(dy, c, y, reverse=False, dtype=np.float64):
+    t = [torch.from_numpy(np.ascontiguousarray(a, dtype=dtype)) for a in (dy, c, y)]
+    return tuple(r.numpy() for r in oracle.bwd_torch(*t, reverse=reverse))
+
+
+IMPLS = [("c", oracle.fwd, oracle.bwd), ("numpy", oracle.fwd_numpy, oracle.bwd_numpy),
+         ("torch", _fwd_torch, _bwd_torch)]
 
 
 def _cases():
@@ -134,18 +147,38 @@ class TestInvariants:
         np.testing.assert_array_equal(y[1, 2], impl[1](x[1, 2], c[1, 2], reverse=reverse))
 
 
-def test_c_and_numpy_restatements_agree():
+def test_the_three_restatements_agree():
     for seed, shape in enumerate([(1, 1), (5, 2), (3, 257), (2, 4, 33)]):
         x, c = _rand(shape, 100 + seed, -1.2, 1.2)
         dy, _ = _rand(shape, 200 + seed)
         for reverse in (False, True):
             for dt in (np.float32, np.float64):
                 y = oracle.fwd(x, c, reverse, dtype=dt)
-                np.testing.assert_array_equal(y, oracle.fwd_numpy(x, c, reverse, dtype=dt))
                 dx, dc = oracle.bwd(dy, c, y, reverse, dtype=dt)
-                dx2, dc2 = oracle.bwd_numpy(dy, c, y, reverse, dtype=dt)
-                np.testing.assert_array_equal(dx, dx2)
-                np.testing.assert_array_equal(dc, dc2)
+                for _, fwd, bwd in IMPLS[1:]:
+                    np.testing.assert_array_equal(y, fwd(x, c, reverse, dtype=dt))
+                    dx2, dc2 = bwd(dy, c, y, reverse, dtype=dt)
+                    np.testing.assert_array_equal(dx, dx2)
+                    np.testing.assert_array_equal(dc, dc2)
+
+
+def test_rows_on_several_threads_give_the_same_bits():
+    """The C loops run rows on OpenMP threads; a row's arithmetic never crosses threads."""
+    x, c = _rand((37, 501), 7, -1.1, 1.1)
+    dy, _ = _rand((37, 501), 8)
+    had = oracle.threads()
+    try:
+        oracle.threads(1)
+        y1 = oracle.fwd(x, c, True, dtype=np.float32)
+        b1 = oracle.bwd(dy, c, y1, True, dtype=np.float32)
+        assert oracle.threads(4) == 4
+        y4 = oracle.fwd(x, c, True, dtype=np.float32)
+        b4 = oracle.bwd(dy, c, y4, True, dtype=np.float32)
+    finally:
+        oracle.threads(had)
+    np.testing.assert_array_equal(y1, y4)
+    np.testing.assert_array_equal(b1[0], b4[0])
+    np.testing.assert_array_equal(b1[1], b4[1])
 
 
 def _explicit_sum_torch(x, c, reverse):
