@@ -5,6 +5,7 @@ passes data pointers, sizes, strides and the current HIP stream; outputs and the
 workspace are allocated here with torch so that they are stream-ordered like any other tensor.
 There is no fallback: if the shared library is missing, every call raises.
 """
+import collections
 import ctypes
 import os
 import threading
@@ -209,9 +210,10 @@ def output_like(t, fake=False):
 
 
 # ---- look-back workspace, one per (device, stream) ---------------------------------------------
-_workspaces = {}
+_workspaces = collections.OrderedDict()  # least recently used first
 _ws_lock = threading.Lock()
 _WS_MIN_BYTES = 1 << 20
+_WS_MAX_KEPT = 16  # (device, stream) pairs whose workspace is kept; a process rarely launches from more
 
 
 def workspace(device, stream_ptr, nbytes):
@@ -224,6 +226,13 @@ def workspace(device, stream_ptr, nbytes):
             size = max(_WS_MIN_BYTES, 1 << (int(nbytes) - 1).bit_length())
             ws = torch.zeros(size, dtype=torch.uint8, device=device)
             _workspaces[key] = ws
+            # Streams come and go (their handles are even reused); the workspaces of the ones not
+            # launched from for longest are dropped.  A dropped buffer goes back to torch's allocator,
+            # which hands it out again in the order of the stream it was allocated on: the one its
+            # kernels were queued on.
+            while len(_workspaces) > _WS_MAX_KEPT:
+                _workspaces.popitem(last=False)
+        _workspaces.move_to_end(key)
         return ws
 
 
@@ -306,7 +315,8 @@ except AttributeError:  # pragma: no cover
     def _raw_stream(index):
         return torch.cuda.current_stream(index).cuda_stream
 
-_need_cache = {}
+_need_cache = collections.OrderedDict()  # (dtype, layout, phase, pass) -> workspace bytes, least recent first
+_NEED_CACHE_MAX = 1024
 
 
 def _workspace_for(t, phase, lay, is_bwd, tun, stream):
@@ -318,6 +328,13 @@ def _workspace_for(t, phase, lay, is_bwd, tun, stream):
         need = lib().linrec_workspace_bytes_dtype(DTYPES[t.dtype], *lay, phase, is_bwd, tun)
         if key is not None:
             _need_cache[key] = need
+            while len(_need_cache) > _NEED_CACHE_MAX:
+                _need_cache.popitem(last=False)
+    elif key is not None:
+        try:
+            _need_cache.move_to_end(key)
+        except KeyError:  # another thread's insertion pushed it out meanwhile
+            pass
     if not need:
         return None, 0
     ws = workspace(t.device, stream, need)

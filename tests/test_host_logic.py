@@ -700,3 +700,34 @@ def test_fake_functions_serve_device_tensors_without_storage():
             assert nat.batched_layout(t) is None and not nat.kept_layout(t)
             assert torch.ops.linrec_amd.linrec_fwd(t, t, False).is_contiguous()
     assert nat.batched_layout(torch.empty(3, 400, 24).transpose(1, 2)) is None  # host tensors take the dense path
+
+
+def test_caches_of_the_binding_stay_bounded(monkeypatch):
+    """One workspace per (device, stream) and one remembered workspace size per layout: both are kept
+    for the most recently used few only, so a long-lived process with many streams and shapes does not
+    grow without bound."""
+    made = []
+
+    def fake_zeros(size, dtype, device):
+        made.append(size)
+        return torch.empty(size, dtype=dtype)
+
+    monkeypatch.setattr(nat.torch, "zeros", fake_zeros)
+    monkeypatch.setattr(nat, "_workspaces", type(nat._workspaces)())
+    dev = torch.device("cuda", 0)
+    for stream in range(3 * nat._WS_MAX_KEPT):
+        nat.workspace(dev, stream, 100)
+        nat.workspace(dev, 0, 100)  # stream 0 stays in use, so it is never the one dropped
+    assert len(nat._workspaces) == nat._WS_MAX_KEPT
+    assert (0, 0) in nat._workspaces and (0, 3 * nat._WS_MAX_KEPT - 1) in nat._workspaces
+    assert made.count(nat._WS_MIN_BYTES) == 3 * nat._WS_MAX_KEPT  # stream 0 was allocated once
+    ws = nat.workspace(dev, 0, nat._WS_MIN_BYTES + 1)  # growing replaces the buffer
+    assert ws.numel() == 2 * nat._WS_MIN_BYTES and len(nat._workspaces) == nat._WS_MAX_KEPT
+
+    monkeypatch.setattr(nat, "_need_cache", type(nat._need_cache)())
+    monkeypatch.setattr(nat, "_NEED_CACHE_MAX", 8)
+    monkeypatch.setattr(nat, "workspace", lambda device, stream, need: torch.empty(need, dtype=torch.uint8))
+    for L in range(4096, 4096 + 40 * 4, 4):
+        t = torch.empty(600, L)
+        nat._workspace_for(t, 0, nat.row_layout(t), False, None, 0)
+    assert len(nat._need_cache) == 8
