@@ -11,7 +11,8 @@
 // With fewer rows a wave is split into G groups of 64/G lanes: the groups share the same 64/G * VEC
 // rows and take consecutive runs of positions, so a workgroup covers fewer rows and more of the
 // scan axis per step, and the launch has G times as many workgroups.  The maps of a wave's groups
-// are scanned across the groups by lane shuffles before the wave's total goes to LDS.
+// of the two halves are composed through a half swap in the vector ALU (lanes_up_32) before the wave's
+// total goes to LDS.  (Four groups of 16 lanes, 64-byte accesses, ran at half the rate.)
 // One pass over the tensors (12 bytes per element forward, 20 backward), no workspace, no workgroup
 // waits for another.  It serves row counts that leave the plain column kernel a wave or less per
 // SIMD and that fill the chip with workgroups of NW waves: (batch, time, channels) data with a few
@@ -30,6 +31,7 @@ namespace linrec {
 
 template <typename T, int VEC, int U, int NW, int G, int MODE, bool DESC>
 __global__ __launch_bounds__(64 * NW) void colblock_kernel(ColumnArgs p) {
+  static_assert(G == 1 || G == 2, "a wave is whole or split into its two halves");
   constexpr int RL = 64 / G;        // lanes of a group: RL * VEC rows per workgroup
   constexpr int STEP = NW * G * U;  // positions per step of the workgroup
   __shared__ float sh_a[2][NW][RL * VEC];
@@ -119,24 +121,17 @@ __global__ __launch_bounds__(64 * NW) void colblock_kernel(ColumnArgs p) {
         }
       }
     }
-    // the groups of a wave: inclusive scan of their maps across the groups, and what precedes each
+    // the two groups of a wave: the upper one's map becomes the map of both; it keeps what precedes it
     Lanes<VEC> ex_a, ex_b;
     if constexpr (G > 1) {
 #pragma unroll
-      for (int d = 1; d < G; d <<= 1) {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const float pa = __shfl_up(ma.v[e], d * RL), pb = __shfl_up(mb.v[e], d * RL);
-          if (grp >= d) {
-            mb.v[e] = fmaf(pb, ma.v[e], mb.v[e]);
-            ma.v[e] = pa * ma.v[e];
-          }
-        }
-      }
-#pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        ex_a.v[e] = __shfl_up(ma.v[e], RL);
-        ex_b.v[e] = __shfl_up(mb.v[e], RL);
+        ex_a.v[e] = lanes_up_32(ma.v[e]);  // the lower group's map, which precedes the upper group's
+        ex_b.v[e] = lanes_up_32(mb.v[e]);
+        if (grp == 1) {
+          mb.v[e] = fmaf(ex_b.v[e], ma.v[e], mb.v[e]);
+          ma.v[e] = ex_a.v[e] * ma.v[e];
+        }
       }
     }
     if (G == 1 || grp == G - 1) {

@@ -80,4 +80,13 @@ __device__ __forceinline__ float shift_down_one_lane(float v, float last) {
   return dpp_move<DPP_WAVE_SHL1, 0xf>(last, v);
 }
 
+// Lanes 32..63 receive the value of the lane 32 below; lanes 0..31 keep their own.  One vector-ALU
+// instruction on gfx950: v_permlane32_swap exchanges the upper half of its first operand with the
+// lower half of its second.
+__device__ __forceinline__ float lanes_up_32(float v) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, unsigned(halves[0]));
+}
+
 }  // namespace linrec
