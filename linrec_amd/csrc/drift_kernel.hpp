@@ -25,14 +25,16 @@
 
 #include <type_traits>
 
-#include "team_kernel.hpp"  // gather_maps, TileArgs, descriptors, completion count
+#include "tile_kernel.hpp"  // TileArgs, descriptors, completion count
 
 namespace linrec {
 
-// The walk.  Wave 0 publishes the map of tile n after the barrier of step n and, at the top of step n, asks
-// for the maps that enter tile n-2 (published by the team mates a whole step ago, so they are there),
-// ahead of its own loads; the words arrive while tile n is scanned, and the value entering tile n-2 is in
-// LDS by the barrier of step n.  Nothing waits for a round trip to another workgroup.
+// The walk.  Wave 0 publishes the map of tile n after the barrier of step n.  At the top of step n the
+// waves ask for the maps that enter tile n-2 (published by the team mates a whole step ago, so they are
+// there), ahead of their own loads: wave w for the 64 tiles from 64 w + 1 tiles back on, a lane each, so a
+// team has up to 64 NW members.  The words arrive while tile n is scanned; every wave composes its share
+// into one map and leaves it in LDS before the barrier of step n, after which every wave composes the
+// shares for itself.  Nothing waits for a round trip to another workgroup.
 //
 // The loop is unrolled three steps deep so that the three tiles in the works (being scanned, and stored
 // one and two steps from now) and the tiles of loaded data change roles without a register being copied.
@@ -40,11 +42,17 @@ namespace linrec {
 template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1>
 __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   static_assert(PF == 1 || PF == 2, "one or two tiles of loads ahead of the scan");
+  static_assert(NW <= 8, "the waves' shares are composed inside half a DPP row");
   constexpr int WAVE_SLOTS = S * 64;
   constexpr int TILE_SLOTS = NW * WAVE_SLOTS;
   __shared__ float sh_a[2][NW];
   __shared__ float sh_b[2][NW];
-  __shared__ float sh_carry[4];  // steps alternate between [0] and [1]; [2] and [3] are the last two tiles'
+  // what the waves collected of the team mates' maps: steps alternate between [0] and [1]; [2] and [3]
+  // are the last two tiles'
+  __shared__ float sh_pa[4][NW];
+  __shared__ float sh_pb[4][NW];
+  __shared__ int sh_fail[4];     // the step (1 for the last two tiles) in which a wave's wait ran out
+  __shared__ float sh_carry[4];  // then: the value computed from the row's own data instead
 
   const int lane = threadIdx.x & 63;
   const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -57,8 +65,9 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   const long long my_rows = team < p.numseq ? (p.numseq - team + teams - 1) / teams : 0;
   const int items = int(my_rows * per_row);
 
-  uint32_t seq = 0;
-  if (wave == 0) seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint32_t seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x < 4) sh_fail[threadIdx.x] = 0;
+  __syncthreads();
   const RowView rv = make_row_view<VEC>(0, 0, p.seqlen);
 
   struct Item {
@@ -85,68 +94,99 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     TileData<S, VEC, MODE> d;  // (what the store still needs of it: the saved outputs, backward)
     TileScan<S, VEC> r;
     Affine before;  // the waves in front of this one
-    Affine total;   // wave 0: the whole tile's map
+    Affine total;   // the whole tile's map
     Item it;
   };
   TileData<S, VEC, MODE> D[3];  // tile n lies in D[n % 3]
   Item DI[3];
   Pending P[3];                 // and becomes P[n % 3]
 
-  float own_out = 0.0f;  // wave 0: value that left this walker's previous tile of the current row
+  float own_out = 0.0f;  // value that left this walker's previous tile of the current row (every wave keeps it)
 
-  // wave 0: the words of the maps in front of tile `it` (lane i: tile t-1-i), asked for ahead of time
+  // This wave's share of the maps in front of tile `it`: lane i holds tile t - 1 - (64 wave + i).
   auto ask = [&](const Item& it, uint64_t& w0, uint64_t& w1) {
     const int t = it.t;
     const int need = t < M - 1 ? t : M - 1;
+    const int i = 64 * wave + lane;
     w0 = 0;
     w1 = 0;
-    if (lane < need) {
+    if (i < need) {
       const uint64_t* desc = p.desc + 2 * ((long long)it.row * K);
-      const long long idx = t - 1 - lane;
+      const long long idx = t - 1 - i;
       w0 = ld_desc(desc + 2 * idx);
       w1 = ld_desc(desc + 2 * idx + 1);
     }
   };
-  // wave 0: the value entering pending tile `q`, from the words asked for (or by polling, or, when that
-  // runs out, from the row's own data)
-  auto resolve = [&](const Pending& q, uint64_t w0, uint64_t w1) -> float {
+  // Before the barrier: the words asked for (asked for again while a team mate is more than two steps
+  // behind) composed into this wave's share, oldest first, and left in LDS.  A wait that runs out is
+  // noted in LDS instead; the workgroup then takes the value from the row's own data.
+  auto collect = [&](const Item& it, uint64_t w0, uint64_t w1, int slot, int token) {
+    const int t = it.t;
+    const int need = t < M - 1 ? t : M - 1;
+    const int mine = need - 64 * wave < 64 ? need - 64 * wave : 64;  // maps this wave holds
+    if (mine <= 0) return;
+    const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
+    for (int polls = 0;; ++polls) {
+      const bool have = lane >= mine || (uint32_t(w0 >> 32) == want && uint32_t(w1 >> 32) == want);
+      if (__ballot(!have) == 0) break;
+      if (polls >= p.spin_limit) {
+        if (lane == 0) {
+          sh_fail[slot] = token;
+          __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+      }
+      __builtin_amdgcn_s_sleep(1);
+      ask(it, w0, w1);
+    }
+    // towards lane 0: inside each row of 16 lanes by DPP, which leaves a row's composition in its lane 0;
+    // then the up to four rows, the highest lanes first
+    float a[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w0)) : 1.0f};
+    float b[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w1)) : 0.0f};
+    scan_step<DPP_ROW_SHL1, 0xf>(a, b);
+    scan_step<DPP_ROW_SHL2, 0xf>(a, b);
+    scan_step<DPP_ROW_SHL4, 0xf>(a, b);
+    scan_step<DPP_ROW_SHL8, 0xf>(a, b);
+    Affine acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
+    if (mine > 16) {
+      Affine far = {read_lane(a[0], 16), read_lane(b[0], 16)};
+      if (mine > 32) far = compose({read_lane(a[0], 32), read_lane(b[0], 32)}, far);
+      if (mine > 48) far = compose({read_lane(a[0], 48), read_lane(b[0], 48)}, far);
+      acc = compose(far, acc);
+    }
+    if (lane == 0) {
+      sh_pa[slot][wave] = acc.a;
+      sh_pb[slot][wave] = acc.b;
+    }
+  };
+  // After the barrier, in every wave alike: the value entering pending tile `q`.
+  auto combine = [&](const Pending& q, int slot, int token) -> float {
     const int t = q.it.t;
     const int need = t < M - 1 ? t : M - 1;
     float carry_in = 0.0f;
     if (t > 0) {
-      Affine acc = {1.0f, 0.0f};
-      bool ok = true;
-      if (need > 0) {
-        const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
-        const bool mine = lane >= need || (uint32_t(w0 >> 32) == want && uint32_t(w1 >> 32) == want);
-        if (__ballot(!mine) == 0) {
-          // lane i holds the map of tile t-1-i: fold them oldest first, towards lane 0
-          float a[1] = {lane < need ? __builtin_bit_cast(float, uint32_t(w0)) : 1.0f};
-          float b[1] = {lane < need ? __builtin_bit_cast(float, uint32_t(w1)) : 0.0f};
-          // (inside each row of 16 lanes by DPP, which leaves a row's composition in its lane 0; then the
-          // up to four rows, the highest lanes first)
-          scan_step<DPP_ROW_SHL1, 0xf>(a, b);
-          scan_step<DPP_ROW_SHL2, 0xf>(a, b);
-          scan_step<DPP_ROW_SHL4, 0xf>(a, b);
-          scan_step<DPP_ROW_SHL8, 0xf>(a, b);
-          acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
-          if (need > 16) {
-            Affine far = {read_lane(a[0], 16), read_lane(b[0], 16)};
-            if (need > 32) far = compose({read_lane(a[0], 32), read_lane(b[0], 32)}, far);
-            if (need > 48) far = compose({read_lane(a[0], 48), read_lane(b[0], 48)}, far);
-            acc = compose(far, acc);
-          }
-        } else {
-          ok = gather_maps(p.desc + 2 * ((long long)q.it.row * K), t, need, seq, lane, p.spin_limit, acc);
+      if (sh_fail[slot] == token) {  // (the same for the whole workgroup)
+        if (wave == 0) {
+          const float c = recompute_entry<VEC, MODE, DESC>(ptrs_of(q.it.row), rv, t * TILE_SLOTS, lane);
+          if (lane == 0) sh_carry[slot] = c;
         }
-      }
-      if (!ok) {
-        if (lane == 0) __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        carry_in = recompute_entry<VEC, MODE, DESC>(ptrs_of(q.it.row), rv, t * TILE_SLOTS, lane);
-      } else if (t < M) {
-        carry_in = acc.b;  // the maps reach back to the row start
+        __syncthreads();
+        carry_in = sh_carry[slot];
+      } else if (need > 0) {
+        const int shares = (need + 63) >> 6;  // wave w's share lies further back than wave w-1's
+        float a[1] = {1.0f}, b[1] = {0.0f};
+        if (lane < shares) {
+          a[0] = sh_pa[slot][lane];
+          b[0] = sh_pb[slot][lane];
+        }
+        if constexpr (NW > 1) scan_step<DPP_ROW_SHL1, 0xf>(a, b);
+        if constexpr (NW > 2) scan_step<DPP_ROW_SHL2, 0xf>(a, b);
+        if constexpr (NW > 4) scan_step<DPP_ROW_SHL4, 0xf>(a, b);
+        const Affine acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
+        // (up to the row start the maps reach back all the way)
+        carry_in = t < M ? acc.b : fmaf(own_out, acc.a, acc.b);
       } else {
-        carry_in = need > 0 ? fmaf(own_out, acc.a, acc.b) : own_out;
+        carry_in = own_out;
       }
     }
     own_out = t == 0 ? q.total.b : fmaf(carry_in, q.total.a, q.total.b);
@@ -176,7 +216,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     constexpr int OLD = (PH + 1) % 3, LD = (PH + PF) % 3;
     __builtin_amdgcn_sched_barrier(0);  // (nothing of this step moves up into the one before)
     uint64_t w0 = 0, w1 = 0;
-    if (wave == 0 && n >= 2) ask(P[OLD].it, w0, w1);
+    if (n >= 2) ask(P[OLD].it, w0, w1);
     __builtin_amdgcn_sched_barrier(0);
     if (prefetch) load_next(D[LD], DI[LD]);
     TileData<S, VEC, MODE>& d = D[PH];
@@ -191,10 +231,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       sh_a[par][wave] = now.r.total.a;
       sh_b[par][wave] = now.r.total.b;
     }
-    if (wave == 0 && n >= 2) {
-      const float cin = resolve(P[OLD], w0, w1);
-      if (lane == 0) sh_carry[par] = cin;
-    }
+    if (n >= 2) collect(P[OLD].it, w0, w1, par, n);
     __syncthreads();
     wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, now.before, now.total);
     if (wave == 0) {
@@ -204,7 +241,10 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
         st_desc(desc + 2 * (long long)it.t + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, now.total.b));
       }
     }
-    if (n >= 2) store_pending(P[OLD], sh_carry[par]);
+    if (n >= 2) {
+      const float tile_in = combine(P[OLD], par, n);
+      store_pending(P[OLD], tile_in);
+    }
     if constexpr (MODE == MODE_BWD) now.d = d;
     now.it = it;
   };
@@ -212,20 +252,18 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   // both are asked for at once, and one barrier serves both.
   auto finish = [&]<int A>(std::integral_constant<int, A>) {
     constexpr int PREV = (A + 2) % 3;
-    if (wave == 0) {
-      uint64_t w0 = 0, w1 = 0, v0 = 0, v1 = 0;
-      if (items >= 2) ask(P[PREV].it, w0, w1);
-      ask(P[A].it, v0, v1);  // (published moments ago: if the words are not there yet, resolve polls for them)
-      if (items >= 2) {
-        const float cin = resolve(P[PREV], w0, w1);
-        if (lane == 0) sh_carry[2] = cin;
-      }
-      const float cin = resolve(P[A], v0, v1);
-      if (lane == 0) sh_carry[3] = cin;
-    }
+    uint64_t w0 = 0, w1 = 0, v0 = 0, v1 = 0;
+    if (items >= 2) ask(P[PREV].it, w0, w1);
+    ask(P[A].it, v0, v1);  // (published moments ago: if the words are not there yet, collect asks again)
+    if (items >= 2) collect(P[PREV].it, w0, w1, 2, 1);
+    collect(P[A].it, v0, v1, 3, 1);
     __syncthreads();
-    if (items >= 2) store_pending(P[PREV], sh_carry[2]);
-    store_pending(P[A], sh_carry[3]);
+    if (items >= 2) {
+      const float tile_in = combine(P[PREV], 2, 1);
+      store_pending(P[PREV], tile_in);
+    }
+    const float tile_in = combine(P[A], 3, 1);
+    store_pending(P[A], tile_in);
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;

@@ -352,23 +352,50 @@ int64_t sweep_team_size(int64_t tiles_per_row, int64_t most = kSweepMaxTeam) {
 // 1024 x 32768 68.3 / 114.0 against 72.9 / 118.8; 2048 x 16384 69.1 / 114.4 against 70.4 / 120.2;
 // 160 x 131072 44.8 / 73.8 against 47.9 / 78.5; 128 x 262144 69.4 / 116.3 against 78.7 / 119.9;
 // forward only: 16 x 1048576 40.3 against 43.5, 64 x 524288 70.0 against 78.0, 32 x 1048576 72.9 against
-// 81.9, 8 x 4194304 75.9 against 84.6, 512 x 262144 260.9 against 279.1.  Left to the others: more than
-// 2048 rows (4096 x 65536 553 / 959 against 548 / 948), and the backward of fewer than 128 rows or of rows
-// longer than 131072 (16 x 1048576 64.4 against 62.0, 64 x 524288 118.9 against 115.3, 512 x 262144 459.7
-// against 450.8), which tiles of 16384 elements serve better and a drift kernel has no registers for.
+// 81.9, 512 x 262144 260.9 against 279.1.  Fewer than 16 rows, where teams of more than 64 come in (against
+// look-back tiles, or the sweep kernels from 6 rows on): 1 x 33554432 73.6 / 120.2 against 101.9 / 142.4,
+// 3 x 8388608 58.2 / 91.7 against 82.4 / 112.2, 4 x 8388608 71.8 / 120.5 against 101.9 / 143.2,
+// 6 x 4194304 56.0 / 91.4 against 62.0 (teams of 64) / 107.9, 8 x 4194304 71.4 / 120.0 against 73.4 (teams of
+// 64) / 135.1.  Left to the others: more than 2048 rows (4096 x 65536 553 / 959 against 548 / 948), and the
+// backward of 16 to 127 rows or of rows longer than 131072 (16 x 1048576 62.8 against 62.0, 32 x 1048576
+// 121.1 against 121.6, 64 x 524288 118.8 against 118.4, 512 x 262144 459.7 against 450.8), where tiles of
+// 16384 elements, which a drift kernel has no registers for, do as well or better.
+//
+// The team for rows of `tiles_per_row` tiles: the divisor of it that keeps most of the chip busy (whole
+// teams only, every team the same number of rows where that is possible), the larger one of equals: the
+// more of a row is in flight at once, the fewer gaps the launch's reading positions leave.  A lane of a
+// wave per team mate: at most 64 a wave.
+int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int64_t resident) {
+  int64_t best = 1;
+  double best_busy = 0.0;
+  for (int64_t team = std::min<int64_t>({int64_t(64) * waves, resident, tiles_per_row}); team >= 1; --team) {
+    if (tiles_per_row % team != 0) continue;
+    const int64_t teams = std::min(q.numseq, resident / team);
+    const int64_t rounds = ceil_div(q.numseq, teams);
+    const double busy = double(q.numseq * team) / double(rounds * resident);
+    if (busy > best_busy + 1e-9) {
+      best = team;
+      best_busy = busy;
+    }
+  }
+  return best;
+}
 // Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
 int drift_slots_for(const Problem& q, int fv) {
   if (q.dtype != LINREC_DTYPE_F32) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
-  if (q.numseq * 64 < q.cus) return 0;  // teams of at most 64 would leave most of the chip idle
   if (q.numseq > q.at(2048)) return 0;
-  if (q.is_bwd && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
+  if (q.is_bwd && q.numseq * 16 >= q.cus && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
   for (int s : {4, 2}) {
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
     const int64_t tiles_per_row = q.seqlen / tile;
-    if (tiles_per_row < kSweepMinTiles || sweep_team_size(tiles_per_row, 64) < kSweepMinTiles) continue;
+    const int64_t team = drift_team_size(q, tiles_per_row, 8, q.cus);
+    if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
+    // the teams have to fill at least half the chip, and every member gets a few tiles (1 x 4194304 in four
+    // steps of 4096 elements: 16.4 / 19.8 us, what look-back tiles take)
+    if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < (s == 4 ? 3 : 4) * q.cus) continue;
     return s;
   }
   return 0;
@@ -746,12 +773,11 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // Every workgroup of the launch has to be resident at once (a walker waits for its team mates, and a
     // workgroup that has not started yet only starts when another one ends): never more than the CUs hold.
     const int64_t resident = int64_t(workgroups_per_cu(id, block, drift || q.is_bwd ? 1 : 2)) * q.cus;
-    // Drift kernels: as much of a row in flight at once as a team can hold (one wave collects a tile's
-    // maps, a lane per team mate: 64 at most), so that the launch's reading positions leave no gaps.
     const int64_t team = tune && tune->tasks > 0
                              ? tune->tasks
-                             : sweep_team_size(tiles_per_row, std::min<int64_t>(drift ? 64 : kSweepMaxTeam, resident));
-    if (team > 64 || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
+                             : drift ? drift_team_size(q, tiles_per_row, waves, resident)
+                                     : sweep_team_size(tiles_per_row, std::min<int64_t>(kSweepMaxTeam, resident));
+    if (team > (drift ? 64 * waves : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
     int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
     if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;

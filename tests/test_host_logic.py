@@ -138,15 +138,19 @@ class TestPlanner:
         assert "drift_w8_s2_MODE_BWD_1" == names[p2b["kernel_id"]]
         p3 = _plan((16384, 2048), reverse=True)
         assert (p3["waves"], p3["slots"], p3["carry"]) == (4, 2, 0) and "FWD_1" in names[p3["kernel_id"]]
-        p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 64 (half a row in flight each) that go from row to row
+        p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 128 (a whole row in flight each) that go from row to row
         assert p4["family"] == nat.FAMILY_DRIFT and p4["carry"] == 1 and p4["workspace_bytes"] > 0
-        assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (64, 256, 128)
+        assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (128, 256, 128)
         p4bw = _plan((16, 1048576), is_bwd=True)  # the backward takes tiles of 16384 elements
         assert (p4bw["family"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_SWEEP, 8, 16, 256, 64)
         p4r = _plan((16, 1048576 + 4))  # a ragged last tile: one team per row
         assert p4r["family"] == nat.FAMILY_TEAM and p4r["grid"] == 16 * p4r["tasks"] and 2 <= p4r["tasks"] <= 64
-        p4b = _plan((2, 1 << 23))  # too few rows for teams of at most 64: one look-back tile per workgroup
-        assert p4b["family"] == nat.FAMILY_TILE and p4b["carry"] == 1 and p4b["grid"] == 2 * p4b["tiles_per_row"]
+        for rows, is_bwd in ((1, False), (2, False), (3, True), (6, True)):
+            # a few very long rows: one team of the whole chip, every wave of a workgroup collecting maps
+            p4b = _plan((rows, 1 << 23), is_bwd=is_bwd)
+            assert p4b["family"] == nat.FAMILY_DRIFT and (p4b["tasks"], p4b["grid"]) == (256, 256), (rows, p4b)
+        p4c = _plan((1, 1 << 20))  # too few tiles to give every workgroup of the chip a few: one look-back tile per workgroup
+        assert p4c["family"] == nat.FAMILY_TILE and p4c["carry"] == 1 and p4c["grid"] == p4c["tiles_per_row"]
         p5 = nat.plan(torch.empty(256, 262144).t())
         assert p5["family"] == nat.FAMILY_COLUMN and p5["vec"] == 2  # 8 bytes of rows per lane
 
@@ -204,7 +208,7 @@ class TestPlanner:
         assert fam((96, 65536), True) == W and fam((16, 1 << 20), True) == W and fam((512, 262144), True) == W
         # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
         assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
-        assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # teams of at most 64 would leave most of the chip idle
+        assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
         # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
         assert slots((4096, 65536)) == 8 and slots((2304, 131072), True) == 8
@@ -233,7 +237,7 @@ class TestPlanner:
         p2 = nat.plan(torch.empty(300, 4096 * 9))                   # whole tiles of 4096 elements only
         assert (p2["family"], p2["slots"], p2["tasks"], p2["tiles_per_row"], p2["grid"]) == (D, 2, 9, 9, 252)
         assert p["family"] == D and (p["tasks"], p["grid"]) == (24, 240)
-        p = nat.plan(torch.empty(40, 8192 * 24), False, True)       # the backward of fewer than 128 rows waits
+        p = nat.plan(torch.empty(40, 8192 * 24), False, True)       # the backward of 16 to 127 rows waits
         assert p["family"] == W and p["tasks"] == 12
 
     def test_few_rows_on_a_strided_scan_axis_are_cut_into_segments(self):
