@@ -284,6 +284,19 @@ int linrec_stream_mix_f32(int reads, int writes, const float* src0, const float*
                           float* dst0, float* dst1, int64_t n, void* stream);
 
 /*
+ * The same traffic with the launch taking its 16 KiB blocks (4096 floats of every stream per workgroup) in
+ * another order than ascending addresses: bits [hold_lo, hold_lo + hold_bits) of the block index (address
+ * bits 14 + hold_lo and up) become the slowest-changing ones, so the blocks in flight at any moment all
+ * agree in them, as the reading positions of a launch do that keeps one workgroup per row of 2^k bytes.
+ * A probe of how the memory system spreads addresses: it is what tells a launch shape with gaps between
+ * its reading positions from a dense one.  hold_bits == 0 is linrec_stream_mix_f32; otherwise n must be
+ * a power of two of whole blocks and the held bits must lie inside the block index.  No counterpart in the
+ * reference.
+ */
+int linrec_stream_mix_order_f32(int reads, int writes, const float* src0, const float* src1, const float* src2,
+                                float* dst0, float* dst1, int64_t n, int hold_lo, int hold_bits, void* stream);
+
+/*
  * Batched matrix transpose on the device: src holds `batch` dense row-major matrices of rows x cols
  * elements of `elem_size` bytes (2 or 4), dst receives the cols x rows transposes, also dense.
  * The binding uses it to bring tensors whose scan axis is the strided one (time-major data) into

@@ -88,6 +88,7 @@ def _declare(lib):
         "linrec_kernel_attrs": (i32, [i32] + [ctypes.POINTER(ctypes.c_int)] * 4),
         "linrec_copy_f32": (i32, [p, p, i64, p]),
         "linrec_stream_mix_f32": (i32, [i32, i32, p, p, p, p, p, i64, p]),
+        "linrec_stream_mix_order_f32": (i32, [i32, i32, p, p, p, p, p, i64, i32, i32, p]),
         "linrec_transpose": (i32, [i32, p, p, i64, i64, i64, p]),
         "linrec_fwd_batched": (i32, [i32, p, p, p, i64, i64, i64, i64, i64, i64, i32, p, sz, tun, p]),
         "linrec_bwd_batched": (i32, [i32, p, p, p, p, p, i64, i64, i64, i64, i64, i64, i32, p, sz, tun, p]),
@@ -547,9 +548,11 @@ def copy(src, dst):
                                     torch.cuda.current_stream(src.device).cuda_stream), "linrec_copy_f32")
 
 
-def stream_mix(srcs, dsts):
+def stream_mix(srcs, dsts, hold=(0, 0)):
     """Sum of the float32 streams `srcs` (0-3 dense tensors) stored to each of `dsts` (0-2): the
-    memory system's rate for that mix of read and write streams, no scan attached."""
+    memory system's rate for that mix of read and write streams, no scan attached.  `hold` = (lo, bits):
+    the launch takes its 16 KiB blocks in an order that keeps those bits of the block index (address bits
+    14 + lo and up) the same among the blocks in flight (needs a power of two of whole blocks)."""
     ts = list(srcs) + list(dsts)
     assert ts and all(t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 for t in ts)
     n = ts[0].numel()
@@ -557,5 +560,6 @@ def stream_mix(srcs, dsts):
     ps = [t.data_ptr() for t in srcs] + [None] * (3 - len(srcs))
     pd = [t.data_ptr() for t in dsts] + [None] * (2 - len(dsts))
     with torch.cuda.device(ts[0].device):
-        check(lib().linrec_stream_mix_f32(len(srcs), len(dsts), *ps, *pd, n,
-                                          torch.cuda.current_stream(ts[0].device).cuda_stream), "linrec_stream_mix_f32")
+        check(lib().linrec_stream_mix_order_f32(len(srcs), len(dsts), *ps, *pd, n, int(hold[0]), int(hold[1]),
+                                                torch.cuda.current_stream(ts[0].device).cuda_stream),
+              "linrec_stream_mix_order_f32")

@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   Item DI[3];
   Pending P[3];                 // and becomes P[n % 3]
 
-  float own_out = 0.0f;  // value that left this walker's previous tile of the current row (every wave keeps it)
+  float own_out = 0.0f;  // value that left this walker's previous tile of the current row (wave 0; every wave in teams of more than 64)
 
   // This wave's share of the maps in front of tile `it`: lane i holds tile t - 1 - (64 wave + i).
   auto ask = [&](const Item& it, uint64_t& w0, uint64_t& w1) {
@@ -117,50 +117,78 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       w1 = ld_desc(desc + 2 * idx + 1);
     }
   };
+  // A team of at most 64: wave 0 holds all the maps and has the value entering the tile in LDS before the
+  // barrier; the others only read it afterwards.  Larger teams: every wave leaves its share in LDS before
+  // the barrier and composes all the shares for itself after it.
+  const bool wide = M > 64;
   // Before the barrier: the words asked for (asked for again while a team mate is more than two steps
-  // behind) composed into this wave's share, oldest first, and left in LDS.  A wait that runs out is
-  // noted in LDS instead; the workgroup then takes the value from the row's own data.
-  auto collect = [&](const Item& it, uint64_t w0, uint64_t w1, int slot, int token) {
+  // behind) composed, oldest first.  A wait that runs out: wave 0 of a team of at most 64 computes the
+  // value from the row's own data on the spot; in a larger team the wave notes it in LDS and the workgroup
+  // does so after the barrier.
+  auto collect = [&](const Pending& q, uint64_t w0, uint64_t w1, int slot, int token) {
+    const Item it = q.it;
     const int t = it.t;
     const int need = t < M - 1 ? t : M - 1;
     const int mine = need - 64 * wave < 64 ? need - 64 * wave : 64;  // maps this wave holds
-    if (mine <= 0) return;
-    const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
-    for (int polls = 0;; ++polls) {
-      const bool have = lane >= mine || (uint32_t(w0 >> 32) == want && uint32_t(w1 >> 32) == want);
-      if (__ballot(!have) == 0) break;
-      if (polls >= p.spin_limit) {
-        if (lane == 0) {
-          sh_fail[slot] = token;
-          __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wide ? mine <= 0 : wave != 0) return;
+    Affine acc = {1.0f, 0.0f};
+    bool ok = true;
+    if (mine > 0) {
+      const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
+      for (int polls = 0;; ++polls) {
+        const bool have = lane >= mine || (uint32_t(w0 >> 32) == want && uint32_t(w1 >> 32) == want);
+        if (__ballot(!have) == 0) break;
+        if (polls >= p.spin_limit) {
+          ok = false;
+          break;
         }
-        return;
+        __builtin_amdgcn_s_sleep(1);
+        ask(it, w0, w1);
       }
-      __builtin_amdgcn_s_sleep(1);
-      ask(it, w0, w1);
+      if (ok) {
+        // towards lane 0: inside each row of 16 lanes by DPP, which leaves a row's composition in its lane
+        // 0; then the up to four rows, the highest lanes first
+        float a[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w0)) : 1.0f};
+        float b[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w1)) : 0.0f};
+        scan_step<DPP_ROW_SHL1, 0xf>(a, b);
+        scan_step<DPP_ROW_SHL2, 0xf>(a, b);
+        scan_step<DPP_ROW_SHL4, 0xf>(a, b);
+        scan_step<DPP_ROW_SHL8, 0xf>(a, b);
+        acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
+        if (mine > 16) {
+          Affine far = {read_lane(a[0], 16), read_lane(b[0], 16)};
+          if (mine > 32) far = compose({read_lane(a[0], 32), read_lane(b[0], 32)}, far);
+          if (mine > 48) far = compose({read_lane(a[0], 48), read_lane(b[0], 48)}, far);
+          acc = compose(far, acc);
+        }
+      } else if (lane == 0) {
+        __hip_atomic_fetch_add(&p.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
-    // towards lane 0: inside each row of 16 lanes by DPP, which leaves a row's composition in its lane 0;
-    // then the up to four rows, the highest lanes first
-    float a[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w0)) : 1.0f};
-    float b[1] = {lane < mine ? __builtin_bit_cast(float, uint32_t(w1)) : 0.0f};
-    scan_step<DPP_ROW_SHL1, 0xf>(a, b);
-    scan_step<DPP_ROW_SHL2, 0xf>(a, b);
-    scan_step<DPP_ROW_SHL4, 0xf>(a, b);
-    scan_step<DPP_ROW_SHL8, 0xf>(a, b);
-    Affine acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
-    if (mine > 16) {
-      Affine far = {read_lane(a[0], 16), read_lane(b[0], 16)};
-      if (mine > 32) far = compose({read_lane(a[0], 32), read_lane(b[0], 32)}, far);
-      if (mine > 48) far = compose({read_lane(a[0], 48), read_lane(b[0], 48)}, far);
-      acc = compose(far, acc);
+    if (wide) {
+      if (lane == 0) {
+        if (ok) {
+          sh_pa[slot][wave] = acc.a;
+          sh_pb[slot][wave] = acc.b;
+        } else {
+          sh_fail[slot] = token;
+        }
+      }
+      return;
     }
-    if (lane == 0) {
-      sh_pa[slot][wave] = acc.a;
-      sh_pb[slot][wave] = acc.b;
+    float carry_in = 0.0f;
+    if (t > 0) {
+      if (!ok) carry_in = recompute_entry<VEC, MODE, DESC>(ptrs_of(it.row), rv, t * TILE_SLOTS, lane);
+      else if (t < M) carry_in = acc.b;  // the maps reach back to the row start
+      else carry_in = need > 0 ? fmaf(own_out, acc.a, acc.b) : own_out;
     }
+    own_out = t == 0 ? q.total.b : fmaf(carry_in, q.total.a, q.total.b);
+    if (lane == 0) sh_carry[slot] = carry_in;
   };
-  // After the barrier, in every wave alike: the value entering pending tile `q`.
+  // After the barrier: the value entering pending tile `q` (in a team of more than 64, composed by every
+  // wave alike from the shares).
   auto combine = [&](const Pending& q, int slot, int token) -> float {
+    if (!wide) return sh_carry[slot];
     const int t = q.it.t;
     const int need = t < M - 1 ? t : M - 1;
     float carry_in = 0.0f;
@@ -172,7 +200,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
         }
         __syncthreads();
         carry_in = sh_carry[slot];
-      } else if (need > 0) {
+      } else {
         const int shares = (need + 63) >> 6;  // wave w's share lies further back than wave w-1's
         float a[1] = {1.0f}, b[1] = {0.0f};
         if (lane < shares) {
@@ -183,10 +211,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
         if constexpr (NW > 2) scan_step<DPP_ROW_SHL2, 0xf>(a, b);
         if constexpr (NW > 4) scan_step<DPP_ROW_SHL4, 0xf>(a, b);
         const Affine acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
-        // (up to the row start the maps reach back all the way)
-        carry_in = t < M ? acc.b : fmaf(own_out, acc.a, acc.b);
-      } else {
-        carry_in = own_out;
+        carry_in = t < M ? acc.b : fmaf(own_out, acc.a, acc.b);  // (up to the row start the maps reach back all the way)
       }
     }
     own_out = t == 0 ? q.total.b : fmaf(carry_in, q.total.a, q.total.b);
@@ -216,7 +241,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     constexpr int OLD = (PH + 1) % 3, LD = (PH + PF) % 3;
     __builtin_amdgcn_sched_barrier(0);  // (nothing of this step moves up into the one before)
     uint64_t w0 = 0, w1 = 0;
-    if (n >= 2) ask(P[OLD].it, w0, w1);
+    if (n >= 2 && (wide || wave == 0)) ask(P[OLD].it, w0, w1);
     __builtin_amdgcn_sched_barrier(0);
     if (prefetch) load_next(D[LD], DI[LD]);
     TileData<S, VEC, MODE>& d = D[PH];
@@ -231,7 +256,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       sh_a[par][wave] = now.r.total.a;
       sh_b[par][wave] = now.r.total.b;
     }
-    if (n >= 2) collect(P[OLD].it, w0, w1, par, n);
+    if (n >= 2) collect(P[OLD], w0, w1, par, n);
     __syncthreads();
     wave_prefixes<NW>(sh_a[par], sh_b[par], wave, lane, now.before, now.total);
     if (wave == 0) {
@@ -253,10 +278,10 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   auto finish = [&]<int A>(std::integral_constant<int, A>) {
     constexpr int PREV = (A + 2) % 3;
     uint64_t w0 = 0, w1 = 0, v0 = 0, v1 = 0;
-    if (items >= 2) ask(P[PREV].it, w0, w1);
-    ask(P[A].it, v0, v1);  // (published moments ago: if the words are not there yet, collect asks again)
-    if (items >= 2) collect(P[PREV].it, w0, w1, 2, 1);
-    collect(P[A].it, v0, v1, 3, 1);
+    if (items >= 2 && (wide || wave == 0)) ask(P[PREV].it, w0, w1);
+    if (wide || wave == 0) ask(P[A].it, v0, v1);  // (published moments ago: if the words are not there yet, collect asks again)
+    if (items >= 2) collect(P[PREV], w0, w1, 2, 1);
+    collect(P[A], v0, v1, 3, 1);
     __syncthreads();
     if (items >= 2) {
       const float tile_in = combine(P[PREV], 2, 1);

@@ -1167,7 +1167,22 @@ struct MixArgs {
   linrec::v4f* dst[2];
   long long n4;
   long long group0;  // first workgroup-sized block of 1024 slots this launch covers
+  int hold_lo, hold_bits, index_bits;  // launch order other than ascending addresses, see mix_block
 };
+
+// The block of 1024 slots workgroup `b` of the launch takes.  With hold_bits > 0 the launch (of 2^index_bits
+// blocks) goes through the blocks in an order that keeps bits [hold_lo, hold_lo + hold_bits) of the block
+// index the same for as long as possible: they become the slowest-changing ones, so the blocks in flight at
+// any moment all agree in them.
+__device__ __forceinline__ long long mix_block(const MixArgs& a, long long b) {
+  if (a.hold_bits <= 0) return a.group0 + b;
+  const int above = a.index_bits - a.hold_lo - a.hold_bits;  // bits of the index above the held ones
+  const long long low = b & ((1ll << a.hold_lo) - 1);
+  const long long rest = b >> a.hold_lo;
+  const long long held = rest >> above;
+  const long long mid = rest & ((1ll << above) - 1);
+  return low | (held << a.hold_lo) | (mid << (a.hold_lo + a.hold_bits));
+}
 
 // R streams in, W streams out, the access pattern of tile_kernel<4, 4, 4, ...>; the loads stay
 // alive when nothing is stored because a store hangs on their (never matching) sum.
@@ -1175,7 +1190,7 @@ struct MixArgs {
 // checks on every access cost a memory-only kernel about 5 % of its rate).
 template <int R, int W, bool CHECK>
 __global__ __launch_bounds__(256) void mix_kernel(MixArgs a) {
-  const long long base = (a.group0 + blockIdx.x) * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);
+  const long long base = mix_block(a, blockIdx.x) * 1024 + (threadIdx.x >> 6) * 256 + (threadIdx.x & 63);
   linrec::v4f acc[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) acc[j] = linrec::v4f{0.0f, 0.0f, 0.0f, 0.0f};
@@ -1514,8 +1529,22 @@ int linrec_copy_f32(const float* src, float* dst, int64_t n, void* stream) {
 
 int linrec_stream_mix_f32(int reads, int writes, const float* src0, const float* src1, const float* src2,
                           float* dst0, float* dst1, int64_t n, void* stream) {
+  return linrec_stream_mix_order_f32(reads, writes, src0, src1, src2, dst0, dst1, n, 0, 0, stream);
+}
+
+int linrec_stream_mix_order_f32(int reads, int writes, const float* src0, const float* src1, const float* src2,
+                                float* dst0, float* dst1, int64_t n, int hold_lo, int hold_bits, void* stream) {
   if (reads < 0 || reads > 3 || writes < 0 || writes > 2 || reads + writes == 0 || n < 0 || (n & 3)) return LINREC_E_INVALID;
+  if (hold_lo < 0 || hold_bits < 0) return LINREC_E_INVALID;
   if (n == 0) return LINREC_OK;
+  int index_bits = 0;
+  if (hold_bits > 0) {
+    // whole blocks of 4096 floats only, a power of two of them, and the held bits inside the index
+    const int64_t blocks = n / 4096;
+    if (n % 4096 != 0 || (blocks & (blocks - 1)) != 0) return LINREC_E_INVALID;
+    while ((int64_t(1) << index_bits) < blocks) ++index_bits;
+    if (hold_lo + hold_bits > index_bits) return LINREC_E_INVALID;
+  }
   const float* srcs[3] = {src0, src1, src2};
   float* dsts[2] = {dst0, dst1};
   MixArgs a{};
@@ -1528,6 +1557,7 @@ int linrec_stream_mix_f32(int reads, int writes, const float* src0, const float*
     a.dst[w] = reinterpret_cast<linrec::v4f*>(dsts[w]);
   }
   a.n4 = n / 4;
+  a.hold_lo = hold_lo; a.hold_bits = hold_bits; a.index_bits = index_bits;
   const long long full = a.n4 / 1024;
   if (full > 2147483647LL) return LINREC_E_TOO_LARGE;
   const void* fn = nullptr;

@@ -5,7 +5,15 @@ time, throughput and difference to a reference) and eval/func_attrs.py:25-60 (re
 report).  Every compiled geometry that can serve the shape is timed with HIP events on rotating
 buffer sets and checked against the library's default choice for that shape.
 
-    python -m linrec_amd.tune --shape 512 65536 [--dtype f32|f16|bf16] [--reverse] [--transposed] [--mixed-phase] [--attrs] [--csv out.csv]
+    python -m linrec_amd.tune --shape 512 65536 [--dtype f32|f16|bf16] [--reverse] [--transposed] [--mixed-phase]
+                              [--only TEXT] [--attrs] [--csv out.csv]
+    python -m linrec_amd.tune --memory-probe [--shape 512 65536]
+
+`--only TEXT` keeps the geometries whose label contains TEXT (one kernel under a profiler).
+`--memory-probe` times no scan at all: the memory-only kernel with a pass's mix of streams (2 in and 1 out,
+3 in and 2 out) over tensors of the given size, its 16 KiB blocks launched in address order and in orders
+that keep some address bits the same among the blocks in flight, which is what a launch with one
+workgroup per row does to the bits that number the block inside the row.
 """
 import argparse
 import csv
@@ -22,6 +30,7 @@ CHAIN_GEOMETRIES = [(4, 2), (4, 4), (8, 2), (8, 4)]
 STREAM_GEOMETRIES = [(4, 4), (8, 2), (8, 4), (16, 2), (8, 8)]
 TEAM_GEOMETRIES = [(4, 2), (4, 4), (8, 2), (8, 4)]
 SWEEP_GEOMETRIES = [(4, 4), (8, 2), (8, 4), (8, 8)]
+DRIFT_GEOMETRIES = [(8, 4), (8, 2), (4, 4)]  # the backward is compiled for 8 waves x 2 slots only
 
 
 def candidates(t):
@@ -50,6 +59,10 @@ def candidates(t):
                 out.append((f"team w{w} s{s} x{team}", nat.Tuning(nat.FAMILY_TEAM, w, s, -1, team)))
         for w, s in SWEEP_GEOMETRIES:
             out.append((f"sweep w{w} s{s}", nat.Tuning(nat.FAMILY_SWEEP, w, s)))
+        for w, s in DRIFT_GEOMETRIES:
+            out.append((f"drift w{w} s{s}", nat.Tuning(nat.FAMILY_DRIFT, w, s)))  # the planner's team size
+            for team in (16, 64, 128, 256):
+                out.append((f"drift w{w} s{s} x{team}", nat.Tuning(nat.FAMILY_DRIFT, w, s, -1, team)))
     else:
         # strided scan axis: rows per lane (access width) x timesteps per batch
         for width in (1, 2, 4, 8):
@@ -84,8 +97,9 @@ DTYPES = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 
 
 def sweep(shape, reverse=False, transposed=False, sets=3, iters=50, warmup=10, device="cuda:0", dtype=torch.float32,
-          mixed_phase=False):
-    """List of dict rows: one per candidate geometry, forward and backward time and GB/s.
+          mixed_phase=False, only=None):
+    """List of dict rows: one per candidate geometry, forward and backward time and GB/s (a pass a
+    geometry is not compiled for is left out of its row).
     `mixed_phase`: the coefficients start one element off the other tensors' 16-byte phase, which
     forces element-sized accesses (the price of the wide accesses, measured)."""
     dev = torch.device(device)
@@ -104,22 +118,66 @@ def sweep(shape, reverse=False, transposed=False, sets=3, iters=50, warmup=10, d
         bufs.append((x, c, dy, y, dx, dc))
     ref_y = nat.fwd(bufs[0][0], bufs[0][1], reverse)
     ref_dx, ref_dc = nat.bwd(bufs[0][2], bufs[0][1], ref_y, reverse)
+    for b in bufs:
+        b[3].copy_(nat.fwd(b[0], b[1], reverse))  # the saved outputs the backward passes are timed on
+    names = nat.kernel_table()
     rows = []
     for label, tun in candidates(bufs[0][0]):
+        if only is not None and only not in label:
+            continue
+        row = {"geometry": label}
         try:
             pl = nat.plan(bufs[0][0], reverse, False, tun)
+            if tun is not None and pl["family"] != tun.family:
+                raise NotImplementedError
             y = nat.fwd(bufs[0][0], bufs[0][1], reverse, tun)
-            dx, dc = nat.bwd(bufs[0][2], bufs[0][1], y, reverse, tun)
+            diff = (y.float() - ref_y.float()).abs().max().item()
+            f = _event_ms(lambda i: nat.fwd(bufs[i % sets][0], bufs[i % sets][1], reverse, tun, out=bufs[i % sets][4]),
+                          iters, warmup)
+            row.update(kernel=names[pl["kernel_id"]], grid=pl["grid"], team=pl["tasks"], fwd_us=f * 1e3,
+                       fwd_GBps=3 * es * n / f / 1e6, fwd_maxabs_vs_default=diff)
         except (RuntimeError, NotImplementedError):
-            continue  # geometry cannot serve this shape
-        diff = max((a.float() - b.float()).abs().max().item() for a, b in ((y, ref_y), (dx, ref_dx), (dc, ref_dc)))
-        f = _event_ms(lambda i: nat.fwd(bufs[i % sets][0], bufs[i % sets][1], reverse, tun, out=bufs[i % sets][3]),
-                      iters, warmup)
-        b = _event_ms(lambda i: nat.bwd(bufs[i % sets][2], bufs[i % sets][1], bufs[i % sets][3], reverse, tun,
-                                        out=(bufs[i % sets][4], bufs[i % sets][5])), iters, warmup)
-        rows.append({"geometry": label, "kernel": nat.kernel_table()[pl["kernel_id"]], "grid": pl["grid"],
-                     "fwd_us": f * 1e3, "fwd_GBps": 3 * es * n / f / 1e6, "bwd_us": b * 1e3, "bwd_GBps": 5 * es * n / b / 1e6,
-                     "maxabs_vs_default": diff})
+            row.update(kernel="-", grid=0, team=0, fwd_us=float("nan"), fwd_GBps=float("nan"), fwd_maxabs_vs_default=float("nan"))
+        try:
+            pl = nat.plan(bufs[0][0], reverse, True, tun)
+            if tun is not None and pl["family"] != tun.family:
+                raise NotImplementedError
+            dx, dc = nat.bwd(bufs[0][2], bufs[0][1], ref_y, reverse, tun)
+            diff = max((a.float() - b.float()).abs().max().item() for a, b in ((dx, ref_dx), (dc, ref_dc)))
+            b = _event_ms(lambda i: nat.bwd(bufs[i % sets][2], bufs[i % sets][1], bufs[i % sets][3], reverse, tun,
+                                            out=(bufs[i % sets][4], bufs[i % sets][5])), iters, warmup)
+            row.update(bwd_kernel=names[pl["kernel_id"]], bwd_team=pl["tasks"], bwd_us=b * 1e3, bwd_GBps=5 * es * n / b / 1e6,
+                       bwd_maxabs_vs_default=diff)
+        except (RuntimeError, NotImplementedError):
+            row.update(bwd_kernel="-", bwd_team=0, bwd_us=float("nan"), bwd_GBps=float("nan"), bwd_maxabs_vs_default=float("nan"))
+        if row["kernel"] != "-" or row["bwd_kernel"] != "-":
+            rows.append(row)
+    return rows
+
+
+def memory_probe(shape, sets=3, iters=40, warmup=8, device="cuda:0"):
+    """Rows of dicts: GB/s of the memory-only kernel for the forward's and the backward's mix of streams
+    over tensors of shape[0] * shape[1] floats (a power of two), blocks launched in address order and with
+    address bits held among the blocks in flight."""
+    dev = torch.device(device)
+    n = shape[0] * shape[1]
+    assert n % 4096 == 0 and (n // 4096) & (n // 4096 - 1) == 0, "a power of two of 16 KiB blocks"
+    index_bits = (n // 4096).bit_length() - 1
+    srcs = [[torch.randn(n, device=dev) for _ in range(3)] for _ in range(sets)]
+    dsts = [[torch.empty(n, device=dev) for _ in range(2)] for _ in range(sets)]
+    row_bits = (shape[1] * 4).bit_length() - 1  # one workgroup per row holds address bits 14 .. row_bits - 1
+    cases = [("address order", (0, 0))]
+    if 14 < row_bits <= 14 + index_bits:
+        cases.append((f"bits 14-{row_bits - 1} held (one workgroup per row of {shape[1]} floats)", (0, row_bits - 14)))
+    for lo, bits in [(1, 3), (1, 1), (2, 1), (3, 1), (4, 1), (5, 1), (6, 1), (7, 1), (8, 1), (9, 1), (3, 4), (6, 3), (8, 3)]:
+        if lo + bits <= index_bits:
+            cases.append((f"bits {14 + lo}-{14 + lo + bits - 1} held" if bits > 1 else f"bit {14 + lo} held", (lo, bits)))
+    rows = []
+    for label, hold in cases:
+        f = _event_ms(lambda i: nat.stream_mix(srcs[i % sets][:2], dsts[i % sets][:1], hold), iters, warmup)
+        b = _event_ms(lambda i: nat.stream_mix(srcs[i % sets], dsts[i % sets], hold), iters, warmup)
+        rows.append({"blocks in flight": label, "2_in_1_out_us": f * 1e3, "2_in_1_out_GBps": 12 * n / f / 1e6,
+                     "3_in_2_out_us": b * 1e3, "3_in_2_out_GBps": 20 * n / b / 1e6})
     return rows
 
 
@@ -136,16 +194,25 @@ def main(argv=None):
     ap.add_argument("--transposed", action="store_true", help="inputs are transposed views (strided scan axis)")
     ap.add_argument("--mixed-phase", action="store_true",
                     help="offset the coefficients by one element: element-sized instead of 16-byte accesses")
+    ap.add_argument("--only", default=None, metavar="TEXT", help="only the geometries whose label contains TEXT")
+    ap.add_argument("--memory-probe", action="store_true",
+                    help="time the memory-only kernel with address bits held among the blocks in flight instead")
     ap.add_argument("--attrs", action="store_true", help="print the register / LDS / scratch table instead")
     ap.add_argument("--csv", default=None)
     a = ap.parse_args(argv)
-    rows = attrs_report() if a.attrs else sweep(tuple(a.shape), a.reverse, a.transposed, dtype=DTYPES[a.dtype], mixed_phase=a.mixed_phase)
+    if a.attrs:
+        rows = attrs_report()
+    elif a.memory_probe:
+        rows = memory_probe(tuple(a.shape))
+    else:
+        rows = sweep(tuple(a.shape), a.reverse, a.transposed, dtype=DTYPES[a.dtype], mixed_phase=a.mixed_phase, only=a.only)
     if not rows:
         sys.exit("nothing to report")
     cols = list(rows[0])
-    print("  ".join(f"{c:>18s}" for c in cols))
+    width = {c: max(len(c), max(len(f"{r[c]:.1f}" if isinstance(r[c], float) else str(r[c])) for r in rows)) for c in cols}
+    print("  ".join(f"{c:>{width[c]}s}" for c in cols))
     for r in rows:
-        print("  ".join(f"{r[c]:18.1f}" if isinstance(r[c], float) else f"{str(r[c]):>18s}" for c in cols))
+        print("  ".join(f"{r[c]:{width[c]}.1f}" if isinstance(r[c], float) else f"{str(r[c]):>{width[c]}s}" for c in cols), flush=True)
     if a.csv:
         with open(a.csv, "w", newline="") as f:
             w = csv.DictWriter(f, fieldnames=cols)
