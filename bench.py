@@ -33,16 +33,16 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     ("C1", "tile_w8_s2_v4_MODE_FWD_0_0"): 3.195e6,
     ("C1", "tile_w8_s2_v4_MODE_BWD_1_0"): 5.362e6,
-    ("C2", "drift_w8_s4_MODE_FWD_0"): 403.73e6,
-    ("C2", "drift_w8_s2_MODE_BWD_1"): 674.56e6,
+    ("C2", "drift_w8_s4_MODE_FWD_0"): 403.83e6,
+    ("C2", "drift_w8_s2_MODE_BWD_1"): 674.74e6,
     ("C2", "stream_w8_s4_MODE_FWD_0"): 402.71e6,
     ("C2", "stream_w8_s4_MODE_BWD_1"): 671.42e6,
     ("C2", "sweep_w8_s4_MODE_BWD_1"): 673.19e6,
     ("C3", "tile_w4_s2_v4_MODE_FWD_1_0"): 402.58e6,
     ("C3", "tile_w4_s2_v4_MODE_BWD_0_0"): 676.67e6,
-    ("C4", "drift_w8_s4_MODE_FWD_0"): 202.22e6,
+    ("C4", "drift_w8_s4_MODE_FWD_0"): 202.32e6,
     ("C4", "sweep_w8_s4_MODE_FWD_0"): 202.13e6,
-    ("C4", "sweep_w8_s8_MODE_BWD_1"): 336.73e6,
+    ("C4", "sweep_w8_s8_MODE_BWD_1"): 336.69e6,
     ("C5", "column_v2_u8_MODE_FWD_0"): 805.12e6,
     ("C5", "column_v2_u8_MODE_BWD_1"): 1340.78e6,
     ("C2", "bf16_stream_w8_s2_MODE_FWD_0"): 201.40e6,
@@ -139,29 +139,44 @@ def cpu_baseline(cfg, host, budget_s=20.0):
     gb = (FWD_BYTES_PER_ELEM + BWD_BYTES_PER_ELEM) * elems / 1e9
     sample = f"fwd+bwd of all {n} rows, timesteps[:{L_s}] of the same inputs"
 
-    t0 = time.perf_counter()
-    y = oracle.fwd_torch(xs, cs, cfg["reverse"])
-    oracle.bwd_torch(dys, cs, y, cfg["reverse"])
-    t_torch = time.perf_counter() - t0
+    def timed(fn, at_least_s):
+        """Average time of one pass; passes are repeated until `at_least_s` seconds have gone by."""
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            spent = time.perf_counter() - t0
+            if spent >= at_least_s:
+                return spent / reps, reps
+
+    def torch_pass():
+        y = oracle.fwd_torch(xs, cs, cfg["reverse"])
+        oracle.bwd_torch(dys, cs, y, cfg["reverse"])
+
     xn, cn, dyn = (t.numpy() for t in (xs, cs, dys))
-    t0 = time.perf_counter()
-    yn = oracle.fwd_numpy(xn, cn, cfg["reverse"], dtype=np.float32)
-    oracle.bwd_numpy(dyn, cn, yn, cfg["reverse"], dtype=np.float32)
-    t_np = time.perf_counter() - t0
+
+    def numpy_pass():
+        yn = oracle.fwd_numpy(xn, cn, cfg["reverse"], dtype=np.float32)
+        oracle.bwd_numpy(dyn, cn, yn, cfg["reverse"], dtype=np.float32)
+
+    def c_pass():
+        yc = oracle.fwd(xn, cn, cfg["reverse"], dtype=np.float32)
+        oracle.bwd(dyn, cn, yc, cfg["reverse"], dtype=np.float32)
+
+    t_torch, r_torch = timed(torch_pass, 0.35 * budget_s)
+    t_np, r_np = timed(numpy_pass, 0.2 * budget_s)
     threads = oracle.threads()
-    t0 = time.perf_counter()
-    yc = oracle.fwd(xn, cn, cfg["reverse"], dtype=np.float32)
-    oracle.bwd(dyn, cn, yc, cfg["reverse"], dtype=np.float32)
-    t_c = time.perf_counter() - t0
+    c_pass()  # (the threads start up outside the timed passes)
+    t_c, r_c = timed(c_pass, 0.15 * budget_s)
     cpus = os.cpu_count()
     return ({"value": gb / t_torch, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-             "sample": f"{sample}, eager-torch loop over timesteps (the reference's host path), {t_torch:.2f} s, "
-                       f"torch.get_num_threads() = {torch.get_num_threads()}, host has {cpus} cpus"},
+             "sample": f"{sample}, eager-torch loop over timesteps (the reference's host path), {r_torch} passes of "
+                       f"{t_torch:.2f} s, torch.get_num_threads() = {torch.get_num_threads()}, host has {cpus} cpus"},
             {"value": gb / t_np, "unit": "GB/s", "cores": 1, "kind": "port",
-             "sample": f"same sample, the same loop in numpy, {t_np:.2f} s"},
+             "sample": f"same sample, the same loop in numpy, {r_np} passes of {t_np:.2f} s"},
             {"value": gb / t_c, "unit": "GB/s", "cores": threads, "kind": "port",
              "sample": f"same sample, sequential C loop per row, rows over {threads} OpenMP threads "
-                       f"(includes dense copies made by the wrapper), {t_c:.2f} s"})
+                       f"(includes the wrapper's allocation of the results), {r_c} passes of {t_c:.3f} s"})
 
 
 def main():
