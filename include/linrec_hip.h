@@ -67,7 +67,8 @@ extern "C" {
 
 #define LINREC_FAMILY_DRIFT 10  /* the SWEEP launch shape with the exchange between team mates off the critical
                                   path: a scanned tile is kept in registers and stored two steps late, by which
-                                  time the value entering it has arrived without anybody waiting.  Tuning as SWEEP */
+                                  time the value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
+                                  teams of up to 64 a wave (512 for 8 waves): beyond 64 every wave collects maps */
 
 /*
  * Per-call tuning override; NULL selects the built-in gfx950 table.
@@ -215,16 +216,19 @@ size_t linrec_workspace_bytes(int64_t numseq, int64_t seqlen, int64_t row_stride
 
 /*
  * The first 16 bytes of a workspace are four uint32: the launch sequence number, the count of
- * tiles whose look-back gave up waiting, and two reserved words.  The second word is the only
- * one a caller may read (after synchronising): non-zero means some earlier launch on this
- * workspace produced invalid results.  The library never resets it.  Always pass the same
+ * waits for another workgroup that ran out, and two reserved words.  The second word is the only
+ * one a caller may read (after synchronising).  A wave whose wait runs out computes what it was
+ * waiting for from the row's own data, so the results of every launch are valid whatever the
+ * count; non-zero only says that launches were slow because other work held part of the device.
+ * The library never resets it.  Always pass the same
  * workspace_bytes for the same workspace: the split into counters and descriptors depends on it.
  * All of that lives in the lower half of the buffer; the upper half is scratch with no life beyond
  * one call (the per-segment maps of LINREC_FAMILY_SEGMENT), kept apart because a descriptor's
  * validity is a bit pattern that scratch values must never imitate.
  *
- * linrec_set_spin_limit: polls a tile spends on one look-back window before it gives up
- * (process-wide; returns the previous value; polls <= 0 only queries).  No counterpart in the
+ * linrec_set_spin_limit: polls a wave spends on one wait for other workgroups' descriptors
+ * before it stops waiting (process-wide; returns the previous value; polls <= 0 only queries;
+ * a limit of 1 makes every such wait run out, which tests use).  No counterpart in the
  * reference.
  */
 int linrec_set_spin_limit(int polls);
