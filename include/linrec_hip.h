@@ -70,6 +70,14 @@ extern "C" {
                                   time the value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
                                   teams of up to 64 a wave (512 for 8 waves): beyond 64 every wave collects maps */
 
+#define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
+                                   of workgroups share a block of rows and take its steps along the scan axis in
+                                   turn; a step's data stays in registers and is stored two steps late, when the
+                                   team mates' maps have arrived.  Tuning: `waves` = waves per workgroup (16 or 8),
+                                   `slots` = positions per run, `carry` = rows per lane, `tasks` = team size (at
+                                   most the waves).  In the plan, `tiles_per_row` = steps of a row, `tasks` = team
+                                   size */
+
 /*
  * Per-call tuning override; NULL selects the built-in gfx950 table.
  * Replaces the keyword options of the reference's launchers

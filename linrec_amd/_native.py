@@ -19,6 +19,7 @@ FAMILY_AUTO, FAMILY_TILE, FAMILY_COLUMN, FAMILY_NAIVE, FAMILY_STREAM, FAMILY_TEA
 FAMILY_SEGMENT = 8
 FAMILY_FLAT = 9
 FAMILY_DRIFT = 10
+FAMILY_COLDRIFT = 11
 
 
 DTYPES = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}  # LINREC_DTYPE_*

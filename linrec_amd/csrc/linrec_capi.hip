@@ -12,6 +12,7 @@
 
 #include "../../include/linrec_hip.h"
 #include "colblock_kernel.hpp"
+#include "coldrift_kernel.hpp"
 #include "column_kernel.hpp"
 #include "flat_kernel.hpp"
 #include "drift_kernel.hpp"
@@ -121,6 +122,15 @@ struct KernelEntry {
   {PFX "colblock_v" #VEC "_u" #U "_g" #G "_" #MODE "_" #DESC,                                  \
    (const void*)&linrec::colblock_kernel<TT, VEC, U, 16, G, linrec::MODE, DESC != 0>, DT,      \
    LINREC_FAMILY_COLUMN, 16, U, VEC, linrec::MODE, DESC, G}
+// Column drift kernels: column blocks in teams along the scan axis (`carry` column: lane groups per wave).
+#define COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE, DESC)                                    \
+  {PFX "coldrift_w" #NW "_v" #VEC "_u" #U "_" #MODE "_" #DESC,                                 \
+   (const void*)&linrec::coldrift_kernel<TT, VEC, U, NW, 1, linrec::MODE, DESC != 0>, DT,      \
+   LINREC_FAMILY_COLDRIFT, NW, U, VEC, linrec::MODE, DESC, 1}
+#define COLDRIFT_FWD_DIRS(TT, DT, PFX, NW, VEC, U)                                             \
+  COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_FWD, 0), COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_FWD, 1)
+#define COLDRIFT_BWD_DIRS(TT, DT, PFX, NW, VEC, U)                                             \
+  COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_BWD, 0), COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_BWD, 1)
 #define COLBLOCK_FWD_DIRS(TT, DT, PFX, VEC, U, G)                                              \
   COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_FWD, 0), COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_FWD, 1)
 #define COLBLOCK_BWD_DIRS(TT, DT, PFX, VEC, U, G)                                              \
@@ -155,6 +165,8 @@ struct KernelEntry {
 #define GROUP_(...) GROUP_ALL_DIRS(__VA_ARGS__)
 #define FLAT_(...) FLAT_ALL_DIRS(__VA_ARGS__)
 #define SEGMENT_(...) SEGMENT_ALL_DIRS(__VA_ARGS__)
+#define COLDRIFT_FWD_(...) COLDRIFT_FWD_DIRS(__VA_ARGS__)
+#define COLDRIFT_BWD_(...) COLDRIFT_BWD_DIRS(__VA_ARGS__)
 #define COLBLOCK_FWD_(...) COLBLOCK_FWD_DIRS(__VA_ARGS__)
 #define COLBLOCK_BWD_(...) COLBLOCK_BWD_DIRS(__VA_ARGS__)
 
@@ -208,6 +220,11 @@ const KernelEntry kKernels[] = {
     // fewer rows: waves split into 2 groups of lanes that share rows (128-byte accesses; 4 groups of 16
     // floats run at half the rate: 4096 x 8192 151.8 / 270.7 us against 101.1 / 168.7 us)
     COLBLOCK_FWD_(F32, 1, 8, 2), COLBLOCK_BWD_(F32, 1, 8, 2), COLBLOCK_FWD_(F32, 2, 8, 2), COLBLOCK_BWD_(F32, 2, 4, 2),
+    // strided scan axis, a few hundred to a few thousand rows: column blocks in teams along the scan axis
+    // (the backward holds three tensors of four steps: runs of 4 positions)
+    COLDRIFT_FWD_(F32, 16, 1, 8), COLDRIFT_BWD_(F32, 16, 1, 4),
+    COLDRIFT_FWD_(F32, 8, 1, 16), COLDRIFT_BWD_(F32, 8, 1, 8), COLDRIFT_BWD_(F32, 8, 1, 16),
+    COLDRIFT_FWD_(F32, 8, 2, 8), COLDRIFT_BWD_(F32, 8, 2, 8),
     // fp16 and bf16 storage (fp32 arithmetic)
     HALF_KERNELS(F16), HALF_KERNELS(BF16),
 };
@@ -218,7 +235,7 @@ int find_kernel(int dtype, int family, int waves, int slots, int vec, int mode, 
     const KernelEntry& k = kKernels[i];
     const bool waves_matter = family == LINREC_FAMILY_TILE || family == LINREC_FAMILY_STREAM ||
                               family == LINREC_FAMILY_TEAM || family == LINREC_FAMILY_SWEEP || family == LINREC_FAMILY_DRIFT || family == LINREC_FAMILY_GROUP ||
-                              family == LINREC_FAMILY_FLAT;
+                              family == LINREC_FAMILY_FLAT || family == LINREC_FAMILY_COLDRIFT;
     if (k.dtype == dtype && k.family == family && k.slots == slots && k.vec == vec && k.mode == mode &&
         k.desc == desc && k.carry == carry && (!waves_matter || k.waves == waves))
       return i;
@@ -559,6 +576,35 @@ int colblock_kernel_for(const Problem& q, int vec, int groups, int want_depth, i
   }
   return -1;
 }
+// Column drift kernels: the team size for `blocks` blocks of rows of `steps` steps each, 0 if the launch
+// would not be worth it: the power of two that fills the chip, every member with at least four steps.
+int64_t coldrift_team(const Problem& q, int64_t blocks, int64_t steps, int64_t resident, int waves) {
+  int64_t team = 1;
+  while (team * 2 <= waves && blocks * team * 2 <= resident && steps >= 8 * team) team *= 2;
+  return team >= 2 && blocks * team * 2 > q.cus ? team : 0;
+}
+// Whether the planner gives this problem (strided scan axis) to the column drift kernels: fp32 rows next to
+// each other, few enough that teams of at least 4 (backward: 2) along the scan axis are what fills the chip,
+// and enough of them that the teams fill three quarters of it.  Measured forward / backward in us against
+// what the table chose before (segments up to 4095 rows, column blocks from there): 4096 x 16384 157.1 / 255.5
+// against 216.3 / 307.1; 2048 x 16384 83.6 / 132.0 against 107.4 / 150.4; 1024 x 32768 forward 95.6 against
+// 110.4 (backward 162.1 against 154.6: left to the segments); 8192 x 4096 backward 126.8 against 142.7 (forward
+// 80.5 against 78.9: left to the column blocks); 3072 x 16384 140.5 / 213.5 against 168.4 / 248.2; 2048 x 4096
+// 25.5 / 36.2 against 40.8 / 54.3; 4096 x 2048 24.9 / 34.3 against 29.5 / 47.7; 512 x 65536 161.3 / 284.5
+// against 112.7 / 149.9 (left to the segments).
+bool coldrift_applies(const Problem& q) {
+  if (q.dtype != LINREC_DTYPE_F32 || q.seqlen < 2048) return false;
+  if (q.row_stride != 1 && q.numseq != 1 && q.rows_per_batch != 1) return false;
+  const int waves = q.is_bwd ? 8 : 16;
+  const int64_t blocks = ceil_div(q.numseq, 64);
+  const int64_t steps = ceil_div(q.seqlen, 128);
+  const int64_t team = coldrift_team(q, blocks, steps, q.cus, waves);
+  // (teams of 16 only where they fill the whole chip: 768 x 32768 forward 91.4 us in 192 workgroups against
+  // 82.6 us for the segments, 1024 x 32768 98.7 against 109.1 us)
+  // (and teams of 2, which gain least: 6144 x 4096 backward 110.6 us in 192 workgroups against 108.3 us for the
+  // column blocks, 8192 x 4096 127.3 against 141.0 us)
+  return team >= (q.is_bwd ? 2 : 4) && (team > 8 || team == 2 ? blocks * team >= q.cus : blocks * team * 4 >= 3 * q.cus);
+}
 // Rows per lane (`want`, or the planner's choice for 0) if the layout allows a block kernel, else 0.
 int colblock_rows_per_lane(const Problem& q, int want) {
   if (q.elem_stride == 1 && q.seqlen != 1) return 0;
@@ -624,7 +670,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     if (q.numseq % q.rows_per_batch) return LINREC_E_INVALID;
     if (q.elem_stride == 1 && q.seqlen != 1) return LINREC_E_UNSUPPORTED;
     if (family != LINREC_FAMILY_AUTO && family != LINREC_FAMILY_COLUMN && family != LINREC_FAMILY_NAIVE &&
-        family != LINREC_FAMILY_SEGMENT)
+        family != LINREC_FAMILY_SEGMENT && family != LINREC_FAMILY_COLDRIFT)
       return LINREC_E_UNSUPPORTED;
   }
   if (family == LINREC_FAMILY_AUTO) {
@@ -658,6 +704,11 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
           family = LINREC_FAMILY_COLUMN;
           use_colblock = g;
         }
+      }
+      // a few hundred to a few thousand rows: column blocks in teams along the scan axis
+      if (coldrift_applies(q)) {
+        family = LINREC_FAMILY_COLDRIFT;
+        use_colblock = 0;
       }
     } else {
       family = LINREC_FAMILY_NAIVE;
@@ -927,6 +978,49 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     return LINREC_OK;
   }
 
+  // Column drift: column blocks in teams along the scan axis (tuning: `waves` = waves per workgroup,
+  // `slots` = positions per run, `carry` = rows per lane, `tasks` = team size).
+  if (family == LINREC_FAMILY_COLDRIFT) {
+    const bool given = tune && tune->family == LINREC_FAMILY_COLDRIFT;
+    const int vec = colblock_rows_per_lane(q, given && tune->carry > 0 ? tune->carry : 1);
+    if (vec == 0) return LINREC_E_UNSUPPORTED;
+    int waves = 0, depth = 0, id = -1;
+    // (waves, positions per run) in the planner's order of preference: forward 16 waves with runs of 8;
+    // the backward holds three tensors of four steps, which 8 waves have the registers for in runs of 16
+    // (4096 x 16384 255.5 us against 266.6 us for 16 waves with runs of 4; forward 167.2 against 157.1 us)
+    const int fwd_shapes[][2] = {{16, 8}, {8, 16}, {8, 8}, {16, 4}};
+    const int bwd_shapes[][2] = {{8, 16}, {16, 4}, {8, 8}, {16, 8}};
+    for (const auto& wd : q.is_bwd ? bwd_shapes : fwd_shapes) {
+      if (given && tune->waves > 0 && wd[0] != tune->waves) continue;
+      if (given && tune->slots > 0 && wd[1] != tune->slots) continue;
+      id = find_kernel(q.dtype, LINREC_FAMILY_COLDRIFT, wd[0], wd[1], vec, mode, desc, 1);
+      if (id >= 0) {
+        waves = wd[0];
+        depth = wd[1];
+        break;
+      }
+    }
+    if (id < 0) return LINREC_E_UNSUPPORTED;
+    const int64_t blocks = ceil_div(ceil_div(q.numseq, vec), 64);
+    const int64_t steps = ceil_div(q.seqlen, int64_t(waves) * depth);
+    // every workgroup of the launch has to be resident at once: team mates take the steps of a block of rows in turn
+    const int64_t resident = int64_t(workgroups_per_cu(id, 64 * waves, 1)) * q.cus;
+    const int64_t team = given && tune->tasks > 0 ? tune->tasks : coldrift_team(q, blocks, steps, resident, waves);
+    // (a wave collects one team mate's map: a team has at most as many members as a workgroup has waves)
+    if (team < 1 || team > waves || team > steps || blocks * team > resident) return LINREC_E_UNSUPPORTED;
+    const int64_t rows_per_block = int64_t(64) * vec;
+    if (blocks * steps * rows_per_block > 2147483647LL) return LINREC_E_TOO_LARGE;
+    out->family = LINREC_FAMILY_COLDRIFT;
+    out->waves = waves; out->slots = depth; out->vec = vec; out->carry = 1;
+    out->tiles_per_row = int32_t(steps);
+    out->tasks = int32_t(team);
+    out->grid = blocks * team;
+    out->block = 64 * waves;
+    out->kernel_id = id;
+    out->workspace_bytes = linrec_workspace_bytes_for_tiles(blocks * steps * rows_per_block);
+    return LINREC_OK;
+  }
+
   // Column block: the waves of a workgroup share rows (tuning: family COLUMN with carry = lane groups per
   // wave, 1, 2 or 4).
   if (family == LINREC_FAMILY_COLUMN && (use_colblock || (tune && tune->family == LINREC_FAMILY_COLUMN && tune->carry >= 1))) {
@@ -1111,6 +1205,26 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
   a.seg_len = 0; a.maps = nullptr; a.segments = 1; a.lanes_per_segment = 0;
   a.rows_per_batch = q.batched() ? q.rows_per_batch : q.numseq;
   a.batch_stride = q.batched() ? q.batch_stride : 0;
+  if (plan.family == LINREC_FAMILY_COLDRIFT) {
+    if (plan.block != 64 * k.waves || plan.tasks < 1 || plan.tasks > k.waves) return LINREC_E_INVALID;  // (what the kernel is compiled for)
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) || workspace_bytes < plan.workspace_bytes)
+      return LINREC_E_WORKSPACE;
+    const WorkspaceLayout lay = workspace_layout(workspace_bytes);
+    const int64_t rows_per_block = int64_t(64) * plan.vec;
+    if (lay.tiles < (plan.grid / plan.tasks) * plan.tiles_per_row * rows_per_block) return LINREC_E_WORKSPACE;
+    linrec::ColDriftArgs d{};
+    d.col = a;
+    d.chain.num_tiles = plan.grid;
+    d.chain.tasks = plan.tasks;
+    d.chain.ws = static_cast<linrec::CarryHeader*>(workspace);
+    d.chain.counters = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + lay.counters_offset);
+    d.chain.desc = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + lay.desc_offset);
+    d.chain.ws_tiles = lay.tiles;
+    d.chain.spin_limit = g_spin_limit;
+    void* dargs[] = {&d};
+    hipError_t e = hipLaunchKernel(k.fn, dim3((unsigned)plan.grid), dim3((unsigned)plan.block), dargs, 0, stream);
+    return e == hipSuccess ? int(hipGetLastError()) : int(e);
+  }
   void* args[] = {&a};
   if (plan.family == LINREC_FAMILY_SEGMENT) {
     const int64_t segments = plan.tiles_per_row;

@@ -18,7 +18,8 @@ CASES = {
     "tile_f32": (1100000, 2048, False, True, torch.float32, "TILE"),
     "flat_f32": (72000000, 30, False, True, torch.float32, "FLAT"),
     "column_f32": (4194304, 520, True, False, torch.float32, "COLUMN"),
-    "segment_f32": (4000, 537000, True, True, torch.float32, "SEGMENT"),
+    "segment_f32": (700, 3100000, True, True, torch.float32, "SEGMENT"),
+    "coldrift_f32": (4000, 537000, True, True, torch.float32, "COLDRIFT"),
     "colblock_f32": (16000, 134300, True, True, torch.float32, "COLUMN"),
     "drift_f32": (20, 1 << 27, False, True, torch.float32, "DRIFT"),  # (its backward: teams that wait, SWEEP)
     "team_f32": (18, (1 << 27) + 12, False, False, torch.float32, "TEAM"),

@@ -294,6 +294,99 @@ def test_column_block_kernels(nat, reverse, dtype):
     assert not torch.isfinite(dx.cpu()[5]).all() and not torch.isfinite(dx.cpu()[77]).all()
 
 
+@pytest.mark.parametrize("reverse", [False, True])
+def test_column_drift_kernels(nat, reverse):
+    """Scan axis strided, teams of workgroups that share a block of 64 rows (128 with two rows per lane) and take
+    its steps along the scan axis in turn, a step stored two of the workgroup's steps late.  Every compiled
+    geometry (waves per workgroup, positions per run, rows per lane) is forced with team sizes from 1 to the
+    number of waves on row lengths around whole steps, on fewer steps than team members allow and on row counts
+    that leave lanes without rows; then the planner's own choice, non-finite values, a batch of time-major
+    matrices, and a poll limit of one."""
+    D = nat.FAMILY_COLDRIFT
+    dev = torch.device("cuda:0")
+    geometries = [(16, 8, 1, False), (16, 4, 1, True), (8, 16, 1, None), (8, 8, 1, True), (8, 8, 2, None)]  # last: pass (None: both)
+    for n, L in [(64, 128), (2, 129), (130, 257), (66, 1000), (1000, 1290), (190, 2048), (34, 5000), (4098, 700)]:
+        x, c, dy = make_inputs((n, L), "uniform", seed=n + L, transposed=True)
+        y_t, dx_t, dc_t = truth(x, c, dy, reverse)
+        xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+        assert xd.stride() == (1, n)
+        for waves, run, v, only_bwd in geometries:
+            if n % v:
+                continue
+            steps = -(-L // (waves * run))
+            blocks = -(-(n // v) // 64)
+            for team in sorted({1, 2, 3, min(waves, steps), min(8, steps)}):
+                if team > steps or blocks * team > 256:
+                    continue
+                tuning = nat.Tuning(D, waves, run, v, team)
+                what = f"{n} x {L} waves={waves} run={run} rows/lane={v} team={team}"
+                y = torch.from_numpy(y_t).float().to(dev).t().contiguous().t() if only_bwd else None
+                if only_bwd is not True:
+                    plan = nat.plan(xd, reverse, False, tuning)
+                    assert (plan["family"], plan["block"], plan["tasks"], plan["grid"], plan["tiles_per_row"]) == (
+                        D, 64 * waves, team, blocks * team, steps), plan
+                    y = nat.fwd(xd, cd, reverse, tuning, out=_nan_like(xd))
+                    torch.cuda.synchronize()
+                    check_close(y, y_t, what + " outputs")
+                if only_bwd is not False:
+                    dx, dc = nat.bwd(dyd, cd, y, reverse, tuning, out=(_nan_like(xd), _nan_like(xd)))
+                    torch.cuda.synchronize()
+                    check_close(dx, dx_t, what + " d_inputs")
+                    check_close(dc, dc_t, what + " d_coeffs")
+        assert nat.gave_up_count() == 0
+    # the planner's own choice, both passes: teams of 8 on 2048 rows
+    x, c, dy = make_inputs((2048, 4100), "sigmoid", seed=5, transposed=True)
+    for is_bwd in (False, True):
+        plan = nat.plan(x.to(dev), reverse, is_bwd)
+        assert (plan["family"], plan["tasks"], plan["grid"]) == (D, 8, 256), plan
+    _run_both(nat, x, c, dy, reverse, None, "transposed 2048 x 4100")
+    # a batch of time-major matrices: 3 x (2100 timesteps x 1344 channels) scanned over time
+    g = torch.Generator().manual_seed(11)
+    xb, cb, dyb = (f((3, 2100, 1344), generator=g) for f in (torch.randn, torch.rand, torch.randn))
+    xv, cv, dyv = (t.to(dev).transpose(1, 2) for t in (xb, cb, dyb))
+    plan = nat.plan(xv, reverse, False)
+    assert plan["family"] == D and plan["grid"] == 63 * plan["tasks"], plan
+    y = nat.fwd(xv, cv, reverse)
+    dx, dc = nat.bwd(dyv, cv, y, reverse)
+    torch.cuda.synchronize()
+    y_t, dx_t, dc_t = truth(xb.transpose(1, 2), cb.transpose(1, 2), dyb.transpose(1, 2), reverse)
+    check_close(y, y_t, "batched outputs")
+    check_close(dx, dx_t, "batched d_inputs")
+    check_close(dc, dc_t, "batched d_coeffs")
+    # a row with non-finite values stays alone with them, in both passes
+    x, c, dy = make_inputs((130, 3000), "uniform", seed=9, transposed=True)
+    x[5, 300] = float("nan")
+    c[77, 10] = float("inf")
+    xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+    y = nat.fwd(xd, cd, reverse, nat.Tuning(D, 16, 8, 1, 4))
+    clean = torch.ones(130, dtype=torch.bool)
+    clean[5] = clean[77] = False
+    assert torch.isfinite(y.cpu()[clean]).all() and not torch.isfinite(y.cpu()[5]).all() and not torch.isfinite(y.cpu()[77]).all()
+    y_clean = torch.where(torch.isfinite(y), y, torch.zeros_like(y))
+    dyd[5, 100] = float("nan")
+    dx, dc = nat.bwd(dyd, cd, y_clean, reverse, nat.Tuning(D, 8, 16, 1, 4))
+    torch.cuda.synchronize()
+    assert torch.isfinite(dx.cpu()[clean]).all() and torch.isfinite(dc.cpu()[clean]).all()
+    assert not torch.isfinite(dx.cpu()[5]).all() and not torch.isfinite(dx.cpu()[77]).all()
+    # a poll limit of one: waits run out, the value entering a step comes from the rows' own data instead
+    x, c, dy = make_inputs((700, 6000), "uniform", seed=3, transposed=True)
+    y_t, dx_t, dc_t = truth(x, c, dy, reverse)
+    xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+    old = nat.lib().linrec_set_spin_limit(1)
+    try:
+        y = nat.fwd(xd, cd, reverse, nat.Tuning(D, 16, 8, 1, 8))
+        dx, dc = nat.bwd(dyd, cd, y, reverse, nat.Tuning(D, 8, 16, 1, 8))
+        torch.cuda.synchronize()
+    finally:
+        nat.lib().linrec_set_spin_limit(old)
+    print("column drift, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
+    check_close(y, y_t, "poll limit 1 outputs")
+    check_close(dx, dx_t, "poll limit 1 d_inputs")
+    check_close(dc, dc_t, "poll limit 1 d_coeffs")
+    for ws in list(nat._workspaces.values()):
+        ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_block_range_row_counts_through_the_operator(nat, seed):
     """Random (batch, time, channels) and (time, channels) tensors whose row counts fall where the
@@ -387,7 +480,8 @@ def test_time_major_data_with_few_rows(nat, reverse, dtype):
     def check(x, c, dy, what, re_laid_out):
         assert nat._few_rows_on_strided_axis(x, nat.row_layout(x), None) == re_laid_out, what
         if not re_laid_out and x.size(-1) >= 256:
-            assert nat.plan(x, reverse)["family"] == nat.FAMILY_SEGMENT, what
+            # (fp32 rows that fill the chip in teams along the scan axis take the column drift kernels)
+            assert nat.plan(x, reverse)["family"] in (nat.FAMILY_SEGMENT, nat.FAMILY_COLDRIFT), what
         y = nat.fwd(x, c, reverse)
         dx, dc = nat.bwd(dy, c, y, reverse)
         torch.cuda.synchronize()
@@ -399,9 +493,10 @@ def test_time_major_data_with_few_rows(nat, reverse, dtype):
         check_close(dx, dx_t, what + " d_inputs", tol)
         check_close(dc, dc_t, what + " d_coeffs", tol)
 
-    for (n, L) in [(64, 5000), (1000, 777), (7, 333), (2048, 4096)]:
+    for (n, L) in [(64, 5000), (1000, 777), (7, 333), (2048, 4096), (2048, 1500)]:
         x, c, dy = (f((L, n), generator=g).to(dtype).to(dev).t() for f in (torch.randn, torch.rand, torch.randn))
         check(x, c, dy, f"transposed {n} x {L}", False)
+        assert (nat.plan(x, reverse)["family"] == nat.FAMILY_COLDRIFT) == ((n, L) == (2048, 4096) and dtype == torch.float32)
     # leading dims that collapse into the rows of one transposed matrix: (L, A, B) seen as (A, B, L)
     x, c, dy = (f((300, 5, 12), generator=g).to(dtype).to(dev).permute(1, 2, 0) for f in (torch.randn, torch.rand, torch.randn))
     check(x, c, dy, "permuted (5, 12, 300)", False)

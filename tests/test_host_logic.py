@@ -243,8 +243,8 @@ class TestPlanner:
     def test_few_rows_on_a_strided_scan_axis_are_cut_into_segments(self):
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
         plan = lambda n, L, **kw: nat.plan(torch.empty(L, n, **kw).t())
-        for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (1024, 100000, 2, 128),
-                                    (4000, 16384, 2, 32), (2048, 4096, 2, 64), (3000, 16384, 2, 43), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
+        for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (700, 100000, 2, 187),
+                                    (3000, 16384, 2, 43), (2048, 1024, 2, 64), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
             p = plan(n, L)
             assert (p["family"], p["vec"], p["tiles_per_row"], p["block"]) == (S, vec, segments, 64), (n, L, p)
             # whole batches of 8 per segment, every position in exactly one segment
@@ -268,13 +268,48 @@ class TestPlanner:
         # rows further apart than one element stay with the element-wise kernel
         assert nat.plan(torch.empty(5000, 128).t()[::2])["family"] == nat.FAMILY_NAIVE
 
+    def test_a_few_thousand_rows_on_a_strided_scan_axis_take_teams_along_the_scan_axis(self):
+        """fp32 rows of at least 2048 elements, few enough that teams of workgroups along the scan axis are what
+        fills the chip: blocks of 64 rows, steps of 128 positions, the team the power of two that fills 256 CUs."""
+        D, S, C = nat.FAMILY_COLDRIFT, nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
+        plan = lambda n, L, bwd=False, **kw: nat.plan(torch.empty(L, n, **kw).t(), False, bwd)
+        names = nat.kernel_table()
+        for n, L, team_f, team_b in [(4096, 16384, 4, 4), (4000, 16384, 4, 4), (2048, 16384, 8, 8), (3072, 16384, 4, 4),
+                                     (2048, 4096, 8, 8), (4096, 2048, 4, 4), (1024, 100000, 16, 0), (8192, 4096, 0, 2),
+                                     (768, 32768, 0, 0), (3000, 16384, 0, 0), (6144, 4096, 0, 0), (512, 65536, 0, 0),
+                                     (4096, 2000, 0, 0)]:
+            for bwd, team in ((False, team_f), (True, team_b)):
+                p = plan(n, L, bwd)
+                if not team:
+                    assert p["family"] in (S, C), (n, L, bwd, p)
+                    continue
+                waves, run = (8, 16) if bwd else (16, 8)
+                assert (p["family"], p["waves"], p["slots"], p["vec"], p["tasks"]) == (D, waves, run, 1, team), (n, L, bwd, p)
+                assert p["grid"] == -(-n // 64) * team <= 256 and p["block"] == 64 * waves
+                assert p["tiles_per_row"] == -(-L // 128) >= 8 * team // 2
+                assert names[p["kernel_id"]] == f"coldrift_w{waves}_v1_u{run}_MODE_{'BWD' if bwd else 'FWD'}_{int(bwd)}"
+                # a descriptor of two 64-bit words per row and step, in the lower half of the workspace
+                assert p["workspace_bytes"] >= 2 * 16 * -(-n // 64) * 64 * p["tiles_per_row"]
+        assert plan(4096, 16384, dtype=torch.bfloat16)["family"] == S   # fp32 only
+        # on request: any compiled geometry, teams of at most as many members as the workgroup has waves
+        x = torch.empty(5000, 700).t()
+        p = nat.plan(x, tuning=nat.Tuning(D, 8, 16, 1, 4))
+        assert (p["family"], p["grid"], p["block"], p["tiles_per_row"]) == (D, 11 * 4, 512, 40)
+        p = nat.plan(x, False, True, nat.Tuning(D, 16, 4, 1, 16))
+        assert (p["grid"], p["block"], p["tiles_per_row"]) == (11 * 16, 1024, 79)
+        for bad in (nat.Tuning(D, 8, 16, 1, 16), nat.Tuning(D, 16, 8, 1, 32), nat.Tuning(D, 16, 16, 1, 2), nat.Tuning(D, 16, 8, 4, 2)):
+            with pytest.raises(NotImplementedError):
+                nat.plan(x, tuning=bad)
+        with pytest.raises(NotImplementedError):
+            nat.plan(torch.empty(700, 5000), tuning=nat.Tuning(D))  # rows along the unit-stride axis
+
     def test_mid_sized_row_counts_on_a_strided_scan_axis_share_rows_among_the_waves_of_a_workgroup(self):
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
         plan = lambda n, L, bwd=False, **kw: nat.plan(torch.empty(L, n, **kw).t(), False, bwd)
         # the block form: plan.carry = lane groups per wave (0 for the plain column kernels)
         block = lambda p: p["carry"] if (p["family"], p["waves"], p["block"], p["workspace_bytes"]) == (C, 16, 1024, 0) else 0
         # the form with the most workgroups that still leaves every CU at most one
-        for n, L, vec, groups in [(4096, 8192, 1, 2), (8192, 4096, 1, 2), (8193, 4096, 1, 1), (12288, 4096, 1, 1),
+        for n, L, vec, groups in [(4096, 1024, 1, 2), (8192, 4096, 1, 2), (8193, 4096, 1, 1), (12288, 4096, 1, 1),
                                   (16384, 2048, 2, 2), (16384, 256, 1, 1), (15358, 2048, 1, 1), (15360, 1024, 2, 2), (16383, 2048, 1, 1),
                                   (16386, 2048, 2, 1), (20000, 2048, 2, 1),
                                   (32768, 2048, 2, 1), (20001, 2048, 1, 1),
@@ -285,12 +320,13 @@ class TestPlanner:
         # the backward with two rows per lane holds three tensors: runs of 4 positions
         assert [(block(p), p["vec"], p["slots"], p["tiles_per_row"]) for p in (plan(24576, 2048, True), plan(32767, 2048, True))] == \
             [(1, 2, 4, 32), (1, 1, 8, 16)]
-        assert block(plan(32768, 2048, True)) == 1 and not block(plan(32770, 2048)) and not block(plan(4095, 4096))
+        assert block(plan(32768, 2048, True)) == 1 and not block(plan(32770, 2048)) and not block(plan(4095, 1024))
         # a second round of workgroups that is at least half full
         assert [block(plan(n, 2048)) for n in (49150, 49152, 61440, 61442)] == [0, 1, 1, 0] and plan(50000, 2048)["vec"] == 2
-        assert plan(4095, 4096)["family"] == S and not block(plan(16384, 255))
+        assert plan(4095, 1024)["family"] == S and not block(plan(16384, 255))
         # the backward with two lane groups from 6144 rows on
-        assert [block(plan(n, 8192, True)) for n in (4096, 6143, 6144, 8192, 8193)] == [0, 0, 2, 2, 1]
+        # (8192 rows: teams of two along the scan axis, the column drift kernels)
+        assert [block(plan(n, 8192, True)) for n in (4096, 6143, 6144, 8192, 8193)] == [0, 0, 2, 0, 1]
         # 16-bit storage: 4 bytes of rows per lane; forward from 8192 rows, backward from 10240, two lane groups
         # up to 16384 rows
         for n, fwd, bwd in [(8190, 0, 0), (8192, 2, 0), (10240, 2, 2), (16384, 2, 2), (16386, 1, 1), (24576, 1, 1), (65536, 1, 1), (65538, 0, 0)]:
