@@ -244,7 +244,7 @@ class TestPlanner:
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
         plan = lambda n, L, **kw: nat.plan(torch.empty(L, n, **kw).t())
         for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (700, 100000, 2, 187),
-                                    (3000, 16384, 2, 43), (2048, 1024, 2, 64), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
+                                    (3000, 16384, 2, 43), (2048, 1024, 2, 32), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
             p = plan(n, L)
             assert (p["family"], p["vec"], p["tiles_per_row"], p["block"]) == (S, vec, segments, 64), (n, L, p)
             # whole batches of 8 per segment, every position in exactly one segment
