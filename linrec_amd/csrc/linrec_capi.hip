@@ -325,6 +325,9 @@ struct Problem {
   // threshold stands for is a number of workgroups or waves per CU.
   int64_t cus = 256;
   int64_t at(int64_t measured_on_256) const { return measured_on_256 * cus / 256; }
+  // The most workspace the caller can give (0: any): the planner leaves out what would need more where
+  // another kernel serves the problem with less.
+  size_t workspace_cap = 0;
   bool batched() const { return rows_per_batch > 0 && rows_per_batch < numseq; }
 };
 
@@ -599,6 +602,8 @@ bool coldrift_applies(const Problem& q) {
   const int64_t blocks = ceil_div(q.numseq, 64);
   const int64_t steps = ceil_div(q.seqlen, 128);
   const int64_t team = coldrift_team(q, blocks, steps, q.cus, waves);
+  // (a caller that can only give so much workspace is served by the kernels that need less)
+  if (q.workspace_cap && linrec_workspace_bytes_for_tiles(blocks * steps * 64) > q.workspace_cap) return false;
   // (teams of 16 only where they fill the whole chip: 768 x 32768 forward 91.4 us in 192 workgroups against
   // 82.6 us for the segments, 1024 x 32768 98.7 against 109.1 us)
   // (and teams of 2, which gain least: 6144 x 4096 backward 110.6 us in 192 workgroups against 108.3 us for the
@@ -1444,13 +1449,15 @@ namespace {
 
 int fwd_impl(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t numseq, int64_t seqlen,
              int64_t row_stride, int64_t elem_stride, int64_t rows_per_batch, int64_t batch_stride, int reverse,
-             void* workspace, size_t workspace_bytes, const linrec_tuning_t* tuning, void* stream) {
+             void* workspace, size_t workspace_bytes, const linrec_tuning_t* tuning, void* stream,
+             size_t workspace_cap = 0) {
   if (numseq < 0 || seqlen < 0 || rows_per_batch < 0) return LINREC_E_INVALID;
   if (dtype < LINREC_DTYPE_F32 || dtype > LINREC_DTYPE_BF16) return LINREC_E_UNSUPPORTED;
   if (numseq == 0 || seqlen == 0) return LINREC_OK;
   if (!inputs || !coeffs || !outputs) return LINREC_E_INVALID;
-  const Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride,
-                                    rows_per_batch, batch_stride, reverse);
+  Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride,
+                              rows_per_batch, batch_stride, reverse);
+  q.workspace_cap = workspace_cap;
   linrec_plan_t plan;
   int rc = make_plan(q, tuning, &plan);
   if (rc != LINREC_OK) return rc;
@@ -1515,20 +1522,22 @@ int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* 
   if (!inputs || !coeffs || !outputs) return LINREC_E_INVALID;
   // What the call needs follows from its arguments alone, so a call that needs more than the static
   // array holds is turned down before anything is enqueued.
-  const Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse);
+  // (kernels that would need more are left out of the choice where another one serves the call with less)
+  Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse);
+  q.workspace_cap = kStaticScratchBytes;
   linrec_plan_t plan;
   const int rc = make_plan(q, tuning, &plan);
   if (rc != LINREC_OK) return rc;
   if (plan.workspace_bytes > kStaticScratchBytes) return LINREC_E_SCRATCH;
   if (plan.workspace_bytes == 0)
     return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, nullptr, 0,
-                    tuning, stream);
+                    tuning, stream, kStaticScratchBytes);
   DeviceState* d = device_state();
   if (!d) return int(hipErrorNoDevice);
   if (!d->scratch_ptr) return d->scratch_rc > 0 ? d->scratch_rc : int(hipErrorInvalidSymbol);
   // The array's size is always passed whole: the split into counters and descriptors depends on it.
   return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, d->scratch_ptr,
-                  kStaticScratchBytes, tuning, stream);
+                  kStaticScratchBytes, tuning, stream, kStaticScratchBytes);
 }
 
 int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void* outputs, void* d_inputs,

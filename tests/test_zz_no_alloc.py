@@ -47,10 +47,11 @@ def _both(x, c, reverse):
 
 def test_noalloc_forward_equals_forward_with_a_workspace_call_after_call():
     # each of these launches keeps state in the scratch: teams that go from row to row (16 rows), look-back
-    # tiles (3 rows, then 1 row), one team per row (8 ragged rows), segments of a strided scan axis
+    # tiles (3 rows, then 1 row), one team per row (8 ragged rows), segments of a strided scan axis, teams along
+    # a strided scan axis (4096 rows)
     cases = [((16, 131072), False, False), ((3, 40000), True, False), ((1, 9000), False, False),
              ((8, 70001), False, False), ((16, 65536), True, False), ((1024, 4096), False, True),
-             ((2, 20000), False, False)]
+             ((4096, 2048), True, True), ((2, 20000), False, False)]
     used_scratch = 0
     for i, (shape, reverse, transposed) in enumerate(cases):
         print("noalloc case", i, shape, reverse, transposed, flush=True)
@@ -59,7 +60,7 @@ def test_noalloc_forward_equals_forward_with_a_workspace_call_after_call():
         used_scratch += need > 0
         assert not torch.isnan(got).any()
         assert torch.equal(want, got), (shape, (want - got).abs().max().item())
-    assert used_scratch >= 6
+    assert used_scratch >= 7
     # the small last case also against the float64 recurrence (bar: 1e-5 normwise, as everywhere)
     truth = oracle.fwd(x.cpu().numpy(), c.cpu().numpy(), False, dtype=np.float64)
     assert oracle.error_report(got.cpu().numpy(), truth)["normwise"] <= 1e-5
@@ -80,3 +81,27 @@ def test_noalloc_forward_of_16_bit_storage_and_kernels_without_scratch():
         want = nat.fwd(x, c)
         torch.cuda.synchronize()
         assert torch.equal(want, got), (dtype, shape)
+
+
+def test_noalloc_takes_another_kernel_where_the_usual_choice_needs_more_scratch_than_there_is():
+    """16384 timesteps x 4096 channels: linrec_fwd takes teams along the scan axis, whose per-step maps need
+    17 MB of workspace; the entry point that allocates nothing serves the call with the kernels that need none
+    instead of turning it down."""
+    lib = nat.lib()
+    x, c = _pair((4096, 16384), 5, transposed=True)
+    lay = nat.row_layout(x)
+    need = lib.linrec_workspace_bytes_dtype(nat.DTYPES[x.dtype], *lay, 0, 0, None)
+    assert nat.plan(x)["family"] == nat.FAMILY_COLDRIFT and need > (4 << 20)
+    got = torch.full_like(x, float("nan"))
+    rc = lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0, None,
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    rows = torch.tensor([0, 1, 63, 64, 2047, 4095], device=x.device)
+    truth = oracle.fwd(x.index_select(0, rows).cpu().numpy(), c.index_select(0, rows).cpu().numpy(), False, dtype=np.float64)
+    assert not torch.isnan(got).any()
+    assert oracle.error_report(got.index_select(0, rows).cpu().numpy(), truth)["normwise"] <= 1e-5
+    # a tuning that insists on the kernel that does not fit is turned down
+    t = nat.Tuning(nat.FAMILY_COLDRIFT)
+    assert lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0,
+                                  ctypes.byref(t), torch.cuda.current_stream().cuda_stream) == -5
