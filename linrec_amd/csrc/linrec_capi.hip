@@ -222,9 +222,8 @@ const KernelEntry kKernels[] = {
     COLBLOCK_FWD_(F32, 1, 8, 2), COLBLOCK_BWD_(F32, 1, 8, 2), COLBLOCK_FWD_(F32, 2, 8, 2), COLBLOCK_BWD_(F32, 2, 4, 2),
     // strided scan axis, a few hundred to a few thousand rows: column blocks in teams along the scan axis
     // (the backward holds three tensors of four steps: runs of 4 positions)
-    COLDRIFT_FWD_(F32, 16, 1, 8), COLDRIFT_BWD_(F32, 16, 1, 4),
-    COLDRIFT_FWD_(F32, 8, 1, 16), COLDRIFT_BWD_(F32, 8, 1, 8), COLDRIFT_BWD_(F32, 8, 1, 16),
-    COLDRIFT_FWD_(F32, 8, 2, 8), COLDRIFT_BWD_(F32, 8, 2, 8),
+    // (two rows per lane and runs of 8 positions in 8 waves were compiled and lost: 4096 x 16384 189 / 276 us)
+    COLDRIFT_FWD_(F32, 16, 1, 8), COLDRIFT_BWD_(F32, 16, 1, 4), COLDRIFT_FWD_(F32, 8, 1, 16), COLDRIFT_BWD_(F32, 8, 1, 16),
     // fp16 and bf16 storage (fp32 arithmetic)
     HALF_KERNELS(F16), HALF_KERNELS(BF16),
 };
@@ -993,8 +992,8 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // (waves, positions per run) in the planner's order of preference: forward 16 waves with runs of 8;
     // the backward holds three tensors of four steps, which 8 waves have the registers for in runs of 16
     // (4096 x 16384 255.5 us against 266.6 us for 16 waves with runs of 4; forward 167.2 against 157.1 us)
-    const int fwd_shapes[][2] = {{16, 8}, {8, 16}, {8, 8}, {16, 4}};
-    const int bwd_shapes[][2] = {{8, 16}, {16, 4}, {8, 8}, {16, 8}};
+    const int fwd_shapes[][2] = {{16, 8}, {8, 16}};
+    const int bwd_shapes[][2] = {{8, 16}, {16, 4}};
     for (const auto& wd : q.is_bwd ? bwd_shapes : fwd_shapes) {
       if (given && tune->waves > 0 && wd[0] != tune->waves) continue;
       if (given && tune->slots > 0 && wd[1] != tune->slots) continue;

@@ -297,7 +297,7 @@ class TestPlanner:
         assert (p["family"], p["grid"], p["block"], p["tiles_per_row"]) == (D, 11 * 4, 512, 40)
         p = nat.plan(x, False, True, nat.Tuning(D, 16, 4, 1, 16))
         assert (p["grid"], p["block"], p["tiles_per_row"]) == (11 * 16, 1024, 79)
-        for bad in (nat.Tuning(D, 8, 16, 1, 16), nat.Tuning(D, 16, 8, 1, 32), nat.Tuning(D, 16, 16, 1, 2), nat.Tuning(D, 16, 8, 4, 2)):
+        for bad in (nat.Tuning(D, 8, 16, 1, 16), nat.Tuning(D, 16, 8, 1, 32), nat.Tuning(D, 16, 16, 1, 2), nat.Tuning(D, 16, 8, 2, 2)):
             with pytest.raises(NotImplementedError):
                 nat.plan(x, tuning=bad)
         with pytest.raises(NotImplementedError):
