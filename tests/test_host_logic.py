@@ -65,6 +65,15 @@ def test_planner_follows_the_compute_unit_count():
             # one team of workgroups per row: never more workgroups than CUs
             t = nat.plan(torch.empty(8, 1048580), False, False)
             assert t["family"] == nat.FAMILY_TEAM and t["grid"] <= cus and t["tasks"] == cus // 8
+            # a single very long row: one team of the whole device
+            w = nat.plan(torch.empty(1, 1 << 25), False, False)
+            assert w["family"] == nat.FAMILY_DRIFT and w["grid"] == w["tasks"] <= cus, (cus, w)
+            # teams along a strided scan axis: whole teams, never more workgroups than CUs
+            for is_bwd in (False, True):
+                c = nat.plan(torch.empty(16384, 4096).t(), False, is_bwd)
+                assert c["grid"] <= max(cus, 64) or c["family"] != nat.FAMILY_COLDRIFT, (cus, c)
+                if c["family"] == nat.FAMILY_COLDRIFT:
+                    assert c["grid"] == 64 * c["tasks"] <= cus
             # one workgroup per row from half the CUs on, teams below
             assert nat.plan(torch.empty(cus // 2 + 1, 65540))["family"] == nat.FAMILY_STREAM
             assert nat.plan(torch.empty(cus // 2, 65540))["family"] == nat.FAMILY_TEAM
@@ -76,6 +85,10 @@ def test_planner_follows_the_compute_unit_count():
             nat.plan(x, False, True, nat.Tuning(nat.FAMILY_SWEEP, 8, 4, 4, 16))
         with pytest.raises(NotImplementedError):
             nat.plan(torch.empty(2, 1048580), False, False, nat.Tuning(nat.FAMILY_TEAM, 8, 4, -1, 16))
+        with pytest.raises(NotImplementedError):
+            nat.plan(torch.empty(16384, 4096).t(), False, False, nat.Tuning(nat.FAMILY_COLDRIFT, 16, 8, 1, 4))
+        with pytest.raises(NotImplementedError):
+            nat.plan(torch.empty(1, 1 << 25), False, False, nat.Tuning(nat.FAMILY_DRIFT, 8, 4, -1, 64))
     finally:
         lib.linrec_set_compute_units(0)
 
