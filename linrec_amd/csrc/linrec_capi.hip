@@ -399,12 +399,22 @@ int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int6
   }
   return best;
 }
+// Many rows with little work for each workgroup (at most four tiles of 8192 elements for each compute unit):
+// filling and draining the three tiles a drift kernel has in the works costs more than the exchange it saves,
+// and the sweep kernels' largest tiles, with the fewest exchanges, do best in both directions.  Forward /
+// backward in us, drift against sweep with tiles of 16384 elements: 96 x 65536 18.4 / 25.9 against 16.6 / 23.4,
+// 128 x 65536 20.1 / 33.2 against 19.9 / 29.4, 120 x 65536 18.9 / 32.4 against 18.6 / 27.9, 150 x 49152
+// 18.1 / 33.3 against 18.4 / 25.7; 200 x 32768 18.2 / 28.5 against 15.2 / 22.3 for one workgroup per row.
+bool little_work_in_many_rows(const Problem& q) {
+  return q.dtype == LINREC_DTYPE_F32 && q.numseq * 4 >= q.cus && q.numseq * q.seqlen <= 4 * 8192 * q.cus;
+}
 // Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
 int drift_slots_for(const Problem& q, int fv) {
   if (q.dtype != LINREC_DTYPE_F32) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
   if (q.numseq > q.at(2048)) return 0;
   if (q.is_bwd && q.numseq * 16 >= q.cus && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
+  if (little_work_in_many_rows(q)) return 0;
   for (int s : {4, 2}) {
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
     const int64_t tile = int64_t(8) * s * 64 * fv;
@@ -438,19 +448,24 @@ int sweep_slots_for(const Problem& q, int fv) {
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0)) return 0;
   const bool half = q.dtype != LINREC_DTYPE_F32;
   int slots = 0;
+  // (little work in many rows: teams of two or three are worth having)
+  const bool little = little_work_in_many_rows(q);
+  const int64_t least_tiles = little ? 2 : kSweepMinTiles;
   for (int s : {8, 4, 2}) {
     if (half && s >= 4) continue;
     // tiles of 16384 elements: the backward pass over fewer rows than the stream kernel takes (fewer
     // exchanges per byte; 16 x 1048576 backward 61.9 against 66.7 us, 64 x 524288 119 against 132 us,
-    // 128 x 262144 121 against 135 us; forward the same or worse, and worse from 512 rows on)
-    if (s == 8 && !(q.is_bwd && q.numseq < q.at(kSweepBelowRows) && q.seqlen / 16384 >= kSweepMinTiles &&
-                    sweep_team_size(q.seqlen / 16384) >= kSweepMinTiles))
+    // 128 x 262144 121 against 135 us; forward the same or worse, and worse from 512 rows on), and both
+    // passes where the rows are many and the work is little
+    if (s == 8 && !((q.is_bwd || little) && q.numseq < q.at(kSweepBelowRows) && q.seqlen / 16384 >= least_tiles &&
+                    sweep_team_size(q.seqlen / 16384) >= least_tiles))
       continue;
     if (q.seqlen % (int64_t(8) * s * 64 * fv) == 0) { slots = s; break; }
   }
   if (slots == 0) return 0;
   const int64_t tiles_per_row = q.seqlen / (int64_t(8) * slots * 64 * fv);
-  if (tiles_per_row < kSweepMinTiles || sweep_team_size(tiles_per_row) < kSweepMinTiles) return 0;
+  const int64_t least = slots == 8 ? least_tiles : kSweepMinTiles;
+  if (tiles_per_row < least || sweep_team_size(tiles_per_row) < least) return 0;
   // 16-bit storage: measured gains only below the stream kernel's row counts (bf16 96 x 65536
   // 12.3 / 17.6 us against 17.5 / 24.7 us for one team per row, 160 x 262144 51 / 101 us against
   // 62 / 121 us; 1000 x 131072 backward 286 us against the stream kernel's 238 us).  Their backward

@@ -636,6 +636,29 @@ def test_rows_beyond_one_per_cu_take_a_second_launch(nat, reverse):
 
 
 @pytest.mark.parametrize("reverse", [False, True])
+def test_little_work_in_many_rows_goes_to_small_teams_with_the_largest_tiles(nat, reverse):
+    """A quarter of the chip's row count and more, at most four tiles of 8192 elements per compute unit: teams that
+    wait, with tiles of 16384 elements, in both directions, teams of two and three among them."""
+    dev = torch.device("cuda:0")
+    for n, L, team in [(100, 32768, 2), (150, 49152, 3), (96, 65536, 4), (64, 131072, 8)]:
+        g = torch.Generator().manual_seed(n)
+        x, c, dy = (torch.randn(n, L, generator=g), torch.rand(n, L, generator=g), torch.randn(n, L, generator=g))
+        xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+        for is_bwd in (False, True):
+            plan = nat.plan(xd, reverse, is_bwd)
+            assert (plan["family"], plan["slots"], plan["tasks"]) == (nat.FAMILY_SWEEP, 8, team), plan
+        y = nat.fwd(xd, cd, reverse)
+        dx, dc = nat.bwd(dyd, cd, y, reverse)
+        torch.cuda.synchronize()
+        y_t, _, _ = truth(x, c, dy, reverse)
+        dx_t, dc_t = oracle.bwd(dy.numpy(), c.numpy(), y.cpu().numpy().astype(np.float64), reverse, dtype=np.float64)
+        check_close(y, y_t, f"{n} x {L} outputs")
+        check_close(dx, dx_t, f"{n} x {L} d_inputs")
+        check_close(dc, dc_t, f"{n} x {L} d_coeffs")
+    assert nat.gave_up_count() == 0
+
+
+@pytest.mark.parametrize("reverse", [False, True])
 def test_broadcast_inputs_get_dense_results(nat, reverse):
     """Expanded tensors (zero strides: a value per row repeated along the scan axis, a row repeated for
     every row, a scalar) are valid inputs; results must not inherit strides under which elements share

@@ -213,9 +213,18 @@ class TestPlanner:
         D, W, ST = nat.FAMILY_DRIFT, nat.FAMILY_SWEEP, nat.FAMILY_STREAM
         # fp32 rows of whole tiles, up to 2048 of them: the forward always, the backward from 128 rows on and
         # for rows up to 131072 elements
-        for shape in [(300, 65536), (96, 65536), (256, 65536), (200, 65536), (512, 65536), (1024, 131072), (2048, 65536),
+        for shape in [(300, 65536), (256, 65536), (200, 65536), (512, 65536), (1024, 131072), (2048, 65536),
                       (16, 1 << 20), (8, 1 << 22), (4, 1 << 20)]:
             assert fam(shape) == D, shape
+        # ... but not where a quarter of the chip's workgroups have a row each and all of them together at most
+        # four tiles of 8192 elements per compute unit: the older kernels fill and drain faster, and the teams
+        # that wait take their largest tiles in both directions, in teams of two if need be
+        assert fam((96, 65536)) == W and fam((200, 32768)) == ST and fam((200, 32768), True) == ST
+        for shape, team in [((128, 65536), 4), ((100, 32768), 2), ((150, 49152), 3), ((64, 131072), 8)]:
+            for bwd in (False, True):
+                q = nat.plan(torch.empty(shape), False, bwd)
+                assert (q["family"], q["slots"], q["tasks"]) == (W, 8, team), (shape, bwd, q)
+        assert fam((130, 65536)) == D and fam((63, 131072)) == D and fam((128, 65536), dtype=torch.bfloat16) == W
         for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 16384)]:
             assert fam(shape, True) == D, shape
         assert fam((96, 65536), True) == W and fam((16, 1 << 20), True) == W and fam((512, 262144), True) == W
