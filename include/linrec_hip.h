@@ -68,7 +68,8 @@ extern "C" {
 #define LINREC_FAMILY_DRIFT 10  /* the SWEEP launch shape with the exchange between team mates off the critical
                                   path: a scanned tile is kept in registers and stored two steps late, by which
                                   time the value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
-                                  teams of up to 64 a wave (512 for 8 waves): beyond 64 every wave collects maps */
+                                  teams of up to 64 a wave (512 for 8 waves): beyond 64 every wave collects maps.
+                                  fp32: 8 waves x 4 or 2 slots forward, 8 x 2 backward; 16-bit storage: 8 x 1, forward */
 
 #define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
                                    of workgroups share a block of rows and take its steps along the scan axis in

@@ -438,8 +438,9 @@ def _validate(first, *rest, names):
 
 
 def gave_up_count(device=None):
-    """Tiles whose look-back hit the poll limit, summed over this process's workspaces on `device`
-    (synchronises).  Non-zero means a launch produced invalid results."""
+    """Waits for another workgroup that hit the poll limit, summed over this process's workspaces on
+    `device` (synchronises).  The results are valid whatever the count (a wave whose wait runs out computes
+    what it was waiting for from the row's own data); non-zero says that launches were slow."""
     total = 0
     with _ws_lock:
         items = list(_workspaces.items())

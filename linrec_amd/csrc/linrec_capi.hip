@@ -177,7 +177,7 @@ struct KernelEntry {
   TILE_(TY, 1, 1, 8, 0), TILE_(TY, 2, 1, 8, 0), TILE_(TY, 4, 1, 8, 0), TILE_(TY, 4, 2, 8, 0),   \
   TILE_(TY, 8, 2, 8, 0), TILE_(TY, 16, 2, 8, 0), TILE_(TY, 4, 2, 8, 1), TILE_(TY, 8, 4, 8, 1),  \
   TILE_(TY, 4, 4, 1, 0), TILE_(TY, 4, 4, 1, 1), STREAM_(TY, 8, 2, 8), TEAM_(TY, 8, 2, 8),       \
-  TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8),                                                  \
+  TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8),                         \
   GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
   COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16),     \
   SEGMENT_(TY, 4, 8), SEGMENT_(TY, 2, 8), SEGMENT_(TY, 1, 8),                             \
@@ -410,12 +410,20 @@ bool little_work_in_many_rows(const Problem& q) {
 }
 // Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
 int drift_slots_for(const Problem& q, int fv) {
-  if (q.dtype != LINREC_DTYPE_F32) return 0;
+  // 16-bit storage: one kernel, forward, tiles of 4096 elements (more per lane do not fit the registers, nor
+  // does any backward).  A step of so little data costs more than the exchange it hides wherever other
+  // kernels fill the chip (bf16 512 x 65536 53 against 37 us, 16 x 1048576 33 against 25 us); one or two very
+  // long rows are what it is for, which no other kernel spreads over every compute unit without waiting
+  // (1 x 33554432 62 against 86 us for look-back tiles, 2 x 16777216 62 against 85 us, 1 x 4194304 14.6
+  // against 16.1 us).
+  const bool half = q.dtype != LINREC_DTYPE_F32;
+  if (half && (q.is_bwd || q.numseq > 2)) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
   if (q.numseq > q.at(2048)) return 0;
   if (q.is_bwd && q.numseq * 16 >= q.cus && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
   if (little_work_in_many_rows(q)) return 0;
-  for (int s : {4, 2}) {
+  for (int s : {4, 2, 1}) {
+    if (half != (s == 1)) continue;
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
@@ -481,6 +489,10 @@ int sweep_slots_for(const Problem& q, int fv) {
 constexpr int64_t kTailMaxRows = 96;  // rows beyond one per CU that a second launch takes (on 256 CUs)
 constexpr int64_t kGroupMaxSlots = 32;  // rows up to this many slots are packed several to a wave
 constexpr int64_t kTeamMinRows = 6;
+// 16-bit storage, forward: teams of 64 already win from three rows on (bf16 3 x 4194304 28.0 against 40.3 us for
+// look-back tiles, 4 x 8388608 55.1 against 85.6 us, 5 x 2097152 21.7 against 35.0 us; the backward is a tie:
+// 3 x 4194304 48.7 against 46.4 us, 4 x 8388608 103.7 against 100.1 us)
+constexpr int64_t kTeamMinRowsHalfFwd = 3;
 
 // Rows one lane of a column kernel takes: 8 bytes' worth (measured best on 262144 x 256: fp32 two
 // rows 131 / 220 us against 132 / 236 us for four; bf16 four rows 70 / 114 us against 101 / 146 us
@@ -710,8 +722,16 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
         if (drift_slots_for(q, fv) > 0) family = LINREC_FAMILY_DRIFT;
         else if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
         else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) family = LINREC_FAMILY_STREAM;
-        else if (q.numseq >= kTeamMinRows) family = LINREC_FAMILY_TEAM;
+        else if (q.numseq >= (half && !q.is_bwd ? kTeamMinRowsHalfFwd : kTeamMinRows)) family = LINREC_FAMILY_TEAM;
       }
+      // 16-bit storage, many rows of exactly two of the stream kernel's tiles (16384 elements): one workgroup of
+      // 8 waves that walks the row beats one tile of 16 waves (bf16 2048 x 16384 34.1 / 57.0 against 36.4 / 59.7 us,
+      // 3000 rows 48.2 / 82.4 against 50.4 / 85.4 us, 4096 rows 64.7 / 112.0 against 68.5 / 118.5 us, 1024 rows
+      // 18.8 / 30.1 against 19.9 / 29.7 us; not rows with a ragged second tile: 2048 x 16000 40.6 / 67.2 against
+      // 35.6 / 60.1 us, 2048 x 12288 33.7 / 53.8 against 29.8 / 46.2 us)
+      if (half && family == LINREC_FAMILY_TILE && q.seqlen == 16384 && q.base_mis == 0 && q.elem_stride == 1 &&
+          q.row_stride % fv == 0 && q.numseq >= q.at(2048))
+        family = LINREC_FAMILY_STREAM;
     } else if (q.row_stride == 1 || q.numseq == 1 || q.rows_per_batch == 1) {
       family = q.numseq < q.at(half ? kSegmentBelowRowsHalf : kSegmentBelowRows) && q.seqlen >= kSegmentMinLen
                    ? LINREC_FAMILY_SEGMENT : LINREC_FAMILY_COLUMN;
@@ -811,7 +831,9 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // 94 / 159 us against 101 / 180 us.  With more rows in the last round, or more rounds, it brings
     // nothing (557 x 60164: 88 / 146 us against 91 / 149 us) or loses (389 x 86108: 87 / 147 us against
     // 83 / 139 us), because the second launch waits for the first.
-    if (!tune && q.numseq > q.cus && q.numseq <= q.cus + q.at(kTailMaxRows))
+    // 16-bit storage: the backward only (bf16 288 x 65536 28.3 / 43.2 us against 27.5 / 46.2 us in one launch,
+    // 352 rows 33.3 / 50.5 us against 28.2 / 48.9 us).
+    if (!tune && q.numseq > q.cus && q.numseq <= q.cus + q.at(kTailMaxRows) && !(half && !q.is_bwd))
       out->tail_rows = int32_t(q.numseq - q.cus);
     size_t tail_workspace = 0;
     if (out->tail_rows) {
@@ -832,7 +854,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     if (q.numseq > 1 && q.row_stride < q.seqlen && q.row_stride > -q.seqlen) return LINREC_E_INVALID;
     const int waves = tune && tune->waves > 0 ? tune->waves : 8;
     const int auto_slots = tune && tune->family != LINREC_FAMILY_AUTO ? 0 : drift ? drift_slots_for(q, fv) : sweep_slots_for(q, fv);
-    const int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? 2 : 4);
+    const int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? (drift ? 1 : 2) : 4);
     const int64_t tile_elems = int64_t(waves) * slots * 64 * fv;
     // every tile of every row has to be a full one
     if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.seqlen % tile_elems != 0) return LINREC_E_UNSUPPORTED;
@@ -1136,8 +1158,9 @@ WorkspaceLayout workspace_layout(size_t whole_bytes) {
   return lay;
 }
 
-// Polls of one look-back window before a tile gives up (about a second of waiting by default).
-int g_spin_limit = 1 << 20;
+// Polls of one look-back window before a tile gives up (about a second of waiting by default).  One value
+// for the process: a wait that runs out costs time, never the result, so no caller depends on another's choice.
+std::atomic<int> g_spin_limit{1 << 20};
 
 #ifdef LINREC_PHASE_TIMING
 unsigned long long* g_timing_buffer = nullptr;
@@ -1191,7 +1214,7 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
       a.desc = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + lay.desc_offset);
       a.ws_tiles = lay.tiles;
     }
-    a.spin_limit = g_spin_limit;
+    a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
 #ifdef LINREC_PHASE_TIMING
     a.timing = g_timing_buffer;
 #endif
@@ -1239,7 +1262,7 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
     d.chain.counters = reinterpret_cast<uint32_t*>(static_cast<char*>(workspace) + lay.counters_offset);
     d.chain.desc = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + lay.desc_offset);
     d.chain.ws_tiles = lay.tiles;
-    d.chain.spin_limit = g_spin_limit;
+    d.chain.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     void* dargs[] = {&d};
     hipError_t e = hipLaunchKernel(k.fn, dim3((unsigned)plan.grid), dim3((unsigned)plan.block), dargs, 0, stream);
     return e == hipSuccess ? int(hipGetLastError()) : int(e);
@@ -1619,9 +1642,8 @@ int linrec_set_compute_units(int cus) {
 int linrec_compute_units(void) { return compute_units(); }
 
 int linrec_set_spin_limit(int polls) {
-  const int old = g_spin_limit;
-  if (polls > 0) g_spin_limit = polls;
-  return old;
+  if (polls > 0) return g_spin_limit.exchange(polls, std::memory_order_relaxed);
+  return g_spin_limit.load(std::memory_order_relaxed);
 }
 
 #ifdef LINREC_PHASE_TIMING

@@ -46,7 +46,7 @@ def _nan_like(t):
     return torch.empty_strided(t.size(), t.stride(), dtype=t.dtype, device=t.device).fill_(float("nan"))
 
 
-def _run(nat, x, c, dy, reverse, tuning, label):
+def _run(nat, x, c, dy, reverse, tuning, label, backward_too=True):
     dev = torch.device("cuda:0")
     xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
     assert xd.stride() == x.stride()
@@ -55,6 +55,9 @@ def _run(nat, x, c, dy, reverse, tuning, label):
     y = nat.fwd(xd, cd, reverse, tuning, out=_nan_like(xd))
     torch.cuda.synchronize()
     _check(y, y_t, x.dtype, f"{label} outputs")
+    if not backward_too:
+        assert nat.gave_up_count() == 0
+        return
     dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y.cpu()), reverse)  # from the 16-bit outputs that were saved
     dx, dc = nat.bwd(dyd, cd, y, reverse, tuning, out=(_nan_like(xd), _nan_like(xd)))
     torch.cuda.synchronize()
@@ -84,6 +87,13 @@ def _tunings(nat, L):
     if L % 8192 == 0:  # rows of whole tiles: teams that go on from row to row
         out.append(nat.Tuning(nat.FAMILY_SWEEP, 8, 2))
         out.append(nat.Tuning(nat.FAMILY_SWEEP, 8, 2, 2, 1))
+    if L % 4096 == 0:  # the same with tiles stored two steps late (compiled for the forward only)
+        k = L // 4096
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1), False))            # team = tiles of a row
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1, 3, 0), False))      # three teams share the rows
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1, 1, 1), False))      # one walker takes whole rows
+        if k % 2 == 0:
+            out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1, 2, k // 2), False))  # two tiles of a row per walker
     return out
 
 
@@ -94,9 +104,12 @@ def test_seqlen_sweep(nat, L, reverse, dtype):
     numseq = 5 if L > 8192 else 33
     x, c, dy = _inputs((numseq, L), dtype, seed=L)
     for tuning in _tunings(nat, L):
+        backward_too = True
+        if isinstance(tuning, tuple):
+            tuning, backward_too = tuning
         label = f"{dtype} L={L} rev={reverse} tune={None if tuning is None else (tuning.family, tuning.waves, tuning.slots, tuning.carry, tuning.tasks)}"
         print(label, flush=True)
-        _run(nat, x, c, dy, reverse, tuning, label)
+        _run(nat, x, c, dy, reverse, tuning, label, backward_too)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
@@ -163,3 +176,33 @@ def test_config_shapes_through_autograd(name, shape, coeffs, reverse, transposed
     dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y), reverse)
     _check(gx, dx_t, dtype, f"{name} d_inputs")
     _check(gc, dc_t, dtype, f"{name} d_coeffs")
+    from linrec_amd import _native
+    assert _native.gave_up_count() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_a_few_very_long_rows(nat, reverse, dtype):
+    """One or two very long rows run forward in teams that fill the launch (four and two collecting waves),
+    three to five rows in teams of up to 64; the backward stays with look-back tiles.  Also with a poll limit
+    of one: every wait of the team members for each other's maps may run out, and the results are the same."""
+    dev = torch.device("cuda:0")
+    for shape, family, team in [((1, 4096 * 1024), nat.FAMILY_DRIFT, 256), ((2, 4096 * 600), nat.FAMILY_DRIFT, 120),
+                                ((3, 4096 * 300), nat.FAMILY_TEAM, 64), ((5, 4096 * 150 + 24), nat.FAMILY_TEAM, 38)]:
+        x, c, dy = _inputs(shape, dtype, seed=shape[0], coeffs="near1")
+        plan = nat.plan(x.to(dev), reverse)
+        assert (plan["family"], plan["tasks"]) == (family, team), plan
+        assert nat.plan(x.to(dev), reverse, True)["family"] == nat.FAMILY_TILE
+        _run(nat, x, c, dy, reverse, None, f"{dtype} {shape} rev={reverse}")
+    x, c, dy = _inputs((1, 4096 * 1024), dtype, seed=7)
+    old = nat.lib().linrec_set_spin_limit(1)
+    try:
+        y = nat.fwd(x.to(dev), c.to(dev), reverse)
+        torch.cuda.synchronize()
+    finally:
+        nat.lib().linrec_set_spin_limit(old)
+    print("16-bit drift, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
+    for ws in list(nat._workspaces.values()):
+        ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
+    f64 = lambda t: t.float().numpy().astype(np.float64)
+    _check(y, oracle.fwd(f64(x), f64(c), reverse), dtype, "with a poll limit of one")

@@ -248,6 +248,20 @@ class TestPlanner:
         assert fam((8, (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
         assert fam((300, 65536), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
         assert fam((16, 1 << 20), dtype=torch.bfloat16) == nat.FAMILY_TEAM
+        # 16-bit storage, forward: one or two very long rows in one team of the whole launch (tiles of 4096
+        # elements), teams of 64 from three rows on; the backward of fewer than six rows stays with look-back tiles
+        for dt in (torch.bfloat16, torch.float16):
+            q = nat.plan(torch.empty(1, 1 << 25, dtype=dt))
+            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 8, 1, 256, 256), q
+            assert fam((2, 1 << 22), dtype=dt) == D and fam((1, 1 << 20), dtype=dt) == nat.FAMILY_TILE
+            assert [fam((n, 1 << 22), dtype=dt) for n in (3, 4, 5, 6)] == [nat.FAMILY_TEAM] * 4
+            assert [fam((n, 1 << 22), True, dtype=dt) for n in (1, 2, 3, 5, 6)] == [nat.FAMILY_TILE] * 4 + [nat.FAMILY_TEAM]
+            # many rows of exactly two of the stream kernel's tiles: one workgroup walks the row
+            assert [fam((n, 16384), b, dtype=dt) for n in (2048, 4096) for b in (False, True)] == [ST] * 4
+            assert fam((1024, 16384), dtype=dt) == nat.FAMILY_TILE and fam((2048, 16000), dtype=dt) == nat.FAMILY_TILE
+            # rows beyond one per CU get a launch of their own in the backward only
+            tails = lambda n: [nat.plan(torch.empty(n, 65536, dtype=dt), False, b)["tail_rows"] for b in (False, True)]
+            assert tails(288) == [0, 32] and tails(352) == [0, 96] and tails(400) == [0, 0]
         # 16-bit backward: one team per row where teams of 256 / rows workgroups fill the chip
         hb = lambda n: fam((n, 262144), True, dtype=torch.bfloat16)
         assert [hb(n) for n in (32, 48, 64, 80, 128)] == [nat.FAMILY_TEAM] * 5
