@@ -225,8 +225,10 @@ class TestPlanner:
                 q = nat.plan(torch.empty(shape), False, bwd)
                 assert (q["family"], q["slots"], q["tasks"]) == (W, 8, team), (shape, bwd, q)
         assert fam((130, 65536)) == D and fam((63, 131072)) == D and fam((128, 65536), dtype=torch.bfloat16) == W
-        for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 16384)]:
+        for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 32768)]:
             assert fam(shape, True) == D, shape
+        # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup each
+        assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST] * 6
         assert fam((96, 65536), True) == W and fam((16, 1 << 20), True) == W and fam((512, 262144), True) == W
         # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
         assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
