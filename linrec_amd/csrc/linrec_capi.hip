@@ -635,11 +635,18 @@ bool coldrift_applies(const Problem& q) {
   const int64_t team = coldrift_team(q, blocks, steps, q.cus, waves);
   // (a caller that can only give so much workspace is served by the kernels that need less)
   if (q.workspace_cap && linrec_workspace_bytes_for_tiles(blocks * steps * 64) > q.workspace_cap) return false;
-  // (teams of 16 only where they fill the whole chip: 768 x 32768 forward 91.4 us in 192 workgroups against
-  // 82.6 us for the segments, 1024 x 32768 98.7 against 109.1 us)
-  // (and teams of 2, which gain least: 6144 x 4096 backward 110.6 us in 192 workgroups against 108.3 us for the
-  // column blocks, 8192 x 4096 127.3 against 141.0 us)
-  return team >= (q.is_bwd ? 2 : 4) && (team > 8 || team == 2 ? blocks * team >= q.cus : blocks * team * 4 >= 3 * q.cus);
+  // Teams of 16 only where they fill seven eighths of the chip: 768 x 32768 forward 91.4 us in 192 workgroups
+  // against 82.6 us for the segments, 900 x 32768 97.6 us in 240 against 117.6 us, 1024 x 32768 98.7 against
+  // 109.1 us.  Teams of 2, which gain least, only where they fill it: 6144 x 4096 backward 110.6 us in 192
+  // workgroups against 108.3 us for the column blocks, 8192 x 4096 127.3 against 141.0 us.  Teams of 4 and 8 from
+  // 65 % on, forward / backward: 1300 x 16384 in 168 workgroups 76.4 / 116.8 us against 86.4 / 128.3 us, 3000 x 8000
+  // in 188 80.5 / 132.0 us against 93.7 / 131.0 us; 2560 x 8192 in 160 70.3 / 102.4 us against 69.5 / 97.7 us,
+  // 1100 x 16384 in 144 74.3 / 107.8 us against 75.7 / 109.9 us, 2200 x 16384 in 140 141.5 / 216.0 us against
+  // 134.9 / 199.6 us.
+  if (team < (q.is_bwd ? 2 : 4)) return false;
+  if (team == 2) return blocks * team >= q.cus;
+  if (team > 8) return blocks * team * 8 >= 7 * q.cus;
+  return blocks * team * 20 >= 13 * q.cus;
 }
 // Rows per lane (`want`, or the planner's choice for 0) if the layout allows a block kernel, else 0.
 int colblock_rows_per_lane(const Problem& q, int want) {

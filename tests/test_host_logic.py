@@ -282,7 +282,7 @@ class TestPlanner:
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
         plan = lambda n, L, **kw: nat.plan(torch.empty(L, n, **kw).t())
         for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (700, 100000, 2, 187),
-                                    (3000, 16384, 2, 43), (2048, 1024, 2, 32), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
+                                    (2200, 16384, 2, 59), (2048, 1024, 2, 32), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
             p = plan(n, L)
             assert (p["family"], p["vec"], p["tiles_per_row"], p["block"]) == (S, vec, segments, 64), (n, L, p)
             # whole batches of 8 per segment, every position in exactly one segment
@@ -314,8 +314,10 @@ class TestPlanner:
         names = nat.kernel_table()
         for n, L, team_f, team_b in [(4096, 16384, 4, 4), (4000, 16384, 4, 4), (2048, 16384, 8, 8), (3072, 16384, 4, 4),
                                      (2048, 4096, 8, 8), (4096, 2048, 4, 4), (1024, 100000, 16, 0), (8192, 4096, 0, 2),
-                                     (768, 32768, 0, 0), (3000, 16384, 0, 0), (6144, 4096, 0, 0), (512, 65536, 0, 0),
-                                     (4096, 2000, 0, 0)]:
+                                     # teams of 4 and 8 from 65 % of the chip on, teams of 16 from seven eighths on
+                                     (3000, 16384, 4, 4), (1300, 16384, 8, 8), (900, 32768, 16, 0),
+                                     (768, 32768, 0, 0), (2560, 8192, 0, 0), (2200, 16384, 0, 0), (6144, 4096, 0, 0),
+                                     (512, 65536, 0, 0), (4096, 2000, 0, 0)]:
             for bwd, team in ((False, team_f), (True, team_b)):
                 p = plan(n, L, bwd)
                 if not team:
