@@ -993,10 +993,18 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
   if (family == LINREC_FAMILY_SEGMENT) {
     if (q.elem_stride == 1 && q.seqlen != 1) return LINREC_E_UNSUPPORTED;
     const bool given = tune && tune->family == LINREC_FAMILY_SEGMENT;
-    // rows per lane: 8 bytes' worth when that leaves at least a wave of lanes, fewer otherwise
+    // rows per lane: 8 bytes' worth when that leaves at least a wave of lanes, fewer otherwise; fp32 from 512
+    // rows on: four rows (16-byte accesses, a wave reads 1 KiB of every position), which the backward likes
+    // (forward / backward in us, four rows against two at their best segment counts: 700 x 100000 278 / 409
+    // against 304 / 465, 2200 x 16384 137 / 191 against 141 / 205, 3000 x 8000 91 / 122 against 96 / 134, 5000 x
+    // 5000 97 / 130 against 97 / 136; 512 x 65536 114 / 157 against 112 / 154, 1024 x 32768 113 / 152 against 109 /
+    // 151; 256 x 65536 62 / 84 against 60 / 83: left at two)
     int vec = given && tune->waves > 0 ? tune->waves : 8 / elem_size_of(q.dtype);
-    if (!(given && tune->waves > 0))
+    if (!(given && tune->waves > 0)) {
+      // (where segments of at least 32 positions of four rows per lane still make all the waves the launch is to have)
+      if (q.dtype == LINREC_DTYPE_F32 && q.numseq / 4 >= q.at(128) && q.numseq * q.seqlen >= 4 * 32 * 64 * segment_waves(q)) vec = 4;
       while (vec > 1 && q.numseq / vec < 64) vec >>= 1;
+    }
     auto rows_fit = [&](int v) {  // v adjacent rows per lane: adjacent in memory, aligned, never across a batch
       return v <= fv && q.row_stride == 1 && q.col_phase % v == 0 && q.elem_stride % v == 0 && q.numseq % v == 0 &&
              (!q.batched() || (q.rows_per_batch % v == 0 && q.batch_stride % v == 0));

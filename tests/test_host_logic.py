@@ -281,8 +281,9 @@ class TestPlanner:
     def test_few_rows_on_a_strided_scan_axis_are_cut_into_segments(self):
         S, C = nat.FAMILY_SEGMENT, nat.FAMILY_COLUMN
         plan = lambda n, L, **kw: nat.plan(torch.empty(L, n, **kw).t())
-        for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (700, 100000, 2, 187),
-                                    (2200, 16384, 2, 59), (2048, 1024, 2, 32), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
+        # (fp32: four rows per lane from 512 rows on where the scan axis is long enough for all the waves wanted)
+        for n, L, vec, segments in [(64, 100000, 1, 962), (256, 65536, 2, 512), (700, 100000, 4, 368),
+                                    (2200, 16384, 4, 114), (2048, 1024, 2, 32), (1000, 300, 2, 10), (72, 460476, 1, 900)]:
             p = plan(n, L)
             assert (p["family"], p["vec"], p["tiles_per_row"], p["block"]) == (S, vec, segments, 64), (n, L, p)
             # whole batches of 8 per segment, every position in exactly one segment
