@@ -249,7 +249,8 @@ int linrec_set_spin_limit(int polls);
  * kernel a CU holds.  Without a device (a plan asked for on a host without a GPU) it assumes the full
  * part's 256.  linrec_compute_units returns the number in use.  linrec_set_compute_units overrides it
  * for the process (tests, planning for another part); 0 returns to asking the device; the previous
- * override is returned, and a negative argument only queries it.
+ * override is returned, and a negative argument only queries it.  A caller that keeps plans or workspace
+ * sizes from one call to the next has to drop them when it changes the override.
  */
 int linrec_compute_units(void);
 int linrec_set_compute_units(int cus);

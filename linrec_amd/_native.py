@@ -317,14 +317,23 @@ except AttributeError:  # pragma: no cover
     def _raw_stream(index):
         return torch.cuda.current_stream(index).cuda_stream
 
-_need_cache = collections.OrderedDict()  # (dtype, layout, phase, pass) -> workspace bytes, least recent first
+_need_cache = collections.OrderedDict()  # (device, dtype, layout, phase, pass) -> workspace bytes, least recent first
 _NEED_CACHE_MAX = 1024
+
+
+def set_compute_units(cus):
+    """Overrides the compute-unit count the planner sizes its launches by (0: ask the device again) and
+    forgets the workspace sizes remembered for the count in force before.  Returns the previous override."""
+    old = lib().linrec_set_compute_units(cus)
+    if cus >= 0:
+        _need_cache.clear()
+    return old
 
 
 def _workspace_for(t, phase, lay, is_bwd, tun, stream):
     """(pointer, bytes) of the workspace this call needs, (None, 0) for kernels without one.
     `phase`: common misalignment of all tensors of the call, -1 if they disagree."""
-    key = (t.dtype, lay, phase, is_bwd) if tun is None else None
+    key = (t.device.index, t.dtype, lay, phase, is_bwd) if tun is None else None
     need = _need_cache.get(key) if key is not None else None
     if need is None:
         need = lib().linrec_workspace_bytes_dtype(DTYPES[t.dtype], *lay, phase, is_bwd, tun)

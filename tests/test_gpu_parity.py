@@ -1070,3 +1070,38 @@ def test_short_rows_keep_nonfinite_values_to_their_row(nat):
             assert torch.equal(got[r], base[r]), r
     assert torch.equal(got[5, :7], base[5, :7]) and not torch.isfinite(got[5, 7:]).any()
     assert torch.equal(got[6, :20], base[6, :20]) and not torch.isfinite(got[6, 20:]).all()
+
+
+@pytest.mark.parametrize("cus", [64, 120])
+def test_grids_sized_for_a_smaller_device_give_the_same_results(nat, cus):
+    """The planner sizes every launch whose workgroups wait for each other by the compute-unit count it was
+    told (here: fewer than the device has, as on a partition of it); teams and grids shrink, the results
+    do not change.  Long rows in teams, a single row in one team, time-major data in teams along the scan axis."""
+    dev = torch.device("cuda:0")
+    lib = nat.lib()
+    assert lib.linrec_set_compute_units(-1) == 0  # no override in force
+    cases = [((96, 65536), False), ((40, 8192 * 24), False), ((5, 4096 * 130), False), ((1, 4096 * 300), False),
+             ((300, 65536 + 4), False), ((1300, 4096), True), ((700, 6000), True)]
+    try:
+        nat.set_compute_units(cus)  # (also forgets the workspace sizes the binding remembers per layout)
+        for shape, transposed in cases:
+            x, c, dy = make_inputs(shape, "uniform", seed=shape[0], transposed=transposed)
+            xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+            assert xd.stride() == x.stride()
+            for reverse in (False, True):
+                pf, pb = nat.plan(xd, reverse, False), nat.plan(xd, reverse, True)
+                print(cus, shape, reverse, "families", pf["family"], pb["family"], "grids", pf["grid"], pb["grid"], flush=True)
+                for p in (pf, pb):
+                    if p["workspace_bytes"] > 0 and p["family"] != nat.FAMILY_TILE and p["family"] != nat.FAMILY_SEGMENT:
+                        assert p["grid"] <= 2 * cus, p  # (at most two workgroups per compute unit, forward sweeps)
+                y = nat.fwd(xd, cd, reverse)
+                dx, dc = nat.bwd(dyd, cd, y, reverse)
+                torch.cuda.synchronize()
+                y_t, _, _ = truth(x, c, dy, reverse)
+                dx_t, dc_t = oracle.bwd(dy.numpy(), c.numpy(), y.cpu().numpy().astype(np.float64), reverse, dtype=np.float64)
+                check_close(y, y_t, f"{cus} CUs {shape} outputs")
+                check_close(dx, dx_t, f"{cus} CUs {shape} d_inputs")
+                check_close(dc, dc_t, f"{cus} CUs {shape} d_coeffs")
+    finally:
+        nat.set_compute_units(0)
+    assert nat.gave_up_count() == 0
