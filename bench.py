@@ -51,8 +51,8 @@ MEASURED_TRAFFIC_BYTES = {
     ("T1", "segment_apply_v2_u8_MODE_FWD_0"): 1352.9e6,
     ("T1", "colblock_v1_u8_g2_MODE_FWD_0"): 805.16e6,
     # column drift kernels: the steps' maps that team mates exchange add 5.5 % forward, 3.3 % backward
-    ("T1", "coldrift_w16_v1_u8_MODE_FWD_0"): 841.37e6,
-    ("T1", "coldrift_w8_v1_u16_MODE_BWD_1"): 1378.26e6,
+    ("T1", "coldrift_w16_v1_u8_MODE_FWD_0"): 849.78e6,
+    ("T1", "coldrift_w8_v1_u16_MODE_BWD_1"): 1387.0e6,
     ("T2", "colblock_v2_u8_g2_MODE_FWD_1"): 402.70e6,
     ("T2", "colblock_v2_u4_g2_MODE_BWD_0"): 670.96e6,
     ("T1", "segment_apply_v2_u8_MODE_BWD_1"): 1889.5e6,

@@ -80,8 +80,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
   if (threadIdx.x < 4) sh_fail[threadIdx.x] = -1;
   __syncthreads();
-  // descriptors: step k of this block of rows: the rows' first words (a) side by side, then their second
-  // words (b), so that a wave's load of either reads one contiguous stretch
+  // descriptors: step k of this block of rows, row i of the block: two words (a, b)
   uint64_t* const desc = ch.desc + 2 * (block * ksteps) * RPB;
 
   struct Batch {
@@ -133,11 +132,11 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
       w.w1[e] = 0;
     }
     if (wave < need) {
-      const uint64_t* d = desc + 2 * (long long)(k - 1 - wave) * RPB + rl;
+      const uint64_t* d = desc + 2 * ((long long)(k - 1 - wave) * RPB + rl * VEC);
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        w.w0[e] = ld_desc(d + e * RL);
-        w.w1[e] = ld_desc(d + RPB + e * RL);
+        w.w0[e] = ld_desc(d + 2 * e);
+        w.w1[e] = ld_desc(d + 2 * e + 1);
       }
     }
   };
@@ -252,11 +251,11 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
         ta.v[e] *= a;
       }
     }
-    uint64_t* d = desc + 2 * (long long)k * RPB + rl;
+    uint64_t* d = desc + 2 * ((long long)k * RPB + rl * VEC);
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-      st_desc(d + e * RL, pack_desc(want, ta.v[e]));
-      st_desc(d + RPB + e * RL, pack_desc(want, tb.v[e]));
+      st_desc(d + 2 * e, pack_desc(want, ta.v[e]));
+      st_desc(d + 2 * e + 1, pack_desc(want, tb.v[e]));
     }
   };
   // After the barrier: pending step in P[PH] (step k of the row, its waves' maps in sh_a/sh_b[PH]) gets the

@@ -111,11 +111,10 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     w0 = 0;
     w1 = 0;
     if (i < need) {
-      // (a row's first words lie side by side, its second words after them: each load reads one stretch)
       const uint64_t* desc = p.desc + 2 * ((long long)it.row * K);
       const long long idx = t - 1 - i;
-      w0 = ld_desc(desc + idx);
-      w1 = ld_desc(desc + K + idx);
+      w0 = ld_desc(desc + 2 * idx);
+      w1 = ld_desc(desc + 2 * idx + 1);
     }
   };
   // A team of at most 64: wave 0 holds all the maps and has the value entering the tile in LDS before the
@@ -263,8 +262,8 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     if (wave == 0) {
       if (lane == 0 && it.t + 1 < K) {
         uint64_t* desc = p.desc + 2 * ((long long)it.row * K);
-        st_desc(desc + it.t, pack_desc((seq << 2) | STATUS_AGGREGATE, now.total.a));
-        st_desc(desc + K + it.t, pack_desc((seq << 2) | STATUS_AGGREGATE, now.total.b));
+        st_desc(desc + 2 * (long long)it.t, pack_desc((seq << 2) | STATUS_AGGREGATE, now.total.a));
+        st_desc(desc + 2 * (long long)it.t + 1, pack_desc((seq << 2) | STATUS_AGGREGATE, now.total.b));
       }
     }
     if (n >= 2) {

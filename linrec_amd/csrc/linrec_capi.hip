@@ -225,7 +225,7 @@ const KernelEntry kKernels[] = {
     // (two rows per lane and runs of 8 positions in 8 waves were compiled and lost: 4096 x 16384 189 / 276 us)
     // (nor two rows per lane with runs of 4 positions in 16 waves, whose 512-byte accesses a memory-only kernel
     // likes better by 14 %: twice the team and half the positions per step make four times the exchange,
-    // 4096 x 16384 forward 173 against 157 us, 2048 x 16384 107.5 against 85.3 us, 8192 x 4096 86.6 against 82.7 us)
+    // 4096 x 16384 forward 187 against 157 us, 2048 x 16384 124 against 85.3 us, 8192 x 4096 89.6 against 82.7 us)
     COLDRIFT_FWD_(F32, 16, 1, 8), COLDRIFT_BWD_(F32, 16, 1, 4), COLDRIFT_FWD_(F32, 8, 1, 16), COLDRIFT_BWD_(F32, 8, 1, 16),
     // fp16 and bf16 storage (fp32 arithmetic)
     HALF_KERNELS(F16), HALF_KERNELS(BF16),
