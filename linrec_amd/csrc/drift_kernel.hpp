@@ -42,7 +42,7 @@ namespace linrec {
 template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1>
 __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   static_assert(PF == 1 || PF == 2, "one or two tiles of loads ahead of the scan");
-  static_assert(NW <= 8, "the waves' shares are composed inside half a DPP row");
+  static_assert(NW <= 16, "the waves' shares are composed inside a DPP row");
   constexpr int WAVE_SLOTS = S * 64;
   constexpr int TILE_SLOTS = NW * WAVE_SLOTS;
   __shared__ float sh_a[2][NW];
@@ -210,6 +210,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
         if constexpr (NW > 1) scan_step<DPP_ROW_SHL1, 0xf>(a, b);
         if constexpr (NW > 2) scan_step<DPP_ROW_SHL2, 0xf>(a, b);
         if constexpr (NW > 4) scan_step<DPP_ROW_SHL4, 0xf>(a, b);
+        if constexpr (NW > 8) scan_step<DPP_ROW_SHL8, 0xf>(a, b);
         const Affine acc = {read_lane(a[0], 0), read_lane(b[0], 0)};
         carry_in = t < M ? acc.b : fmaf(own_out, acc.a, acc.b);  // (up to the row start the maps reach back all the way)
       }

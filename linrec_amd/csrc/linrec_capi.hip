@@ -79,7 +79,7 @@ struct KernelEntry {
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, 2>, DT, LINREC_FAMILY_DRIFT, \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, ((NW) > 8 ? 4 : 2)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
@@ -205,6 +205,7 @@ const KernelEntry kKernels[] = {
     SWEEP_(F32, 8, 4, 4), SWEEP_(F32, 8, 2, 4), SWEEP_(F32, 4, 4, 4), SWEEP_(F32, 8, 8, 4),
     // the same launch shape with a tile stored two steps late, so that nobody waits for the exchange
     DRIFT_FWD_(F32, 8, 4, 4), DRIFT_FWD_(F32, 8, 2, 4), DRIFT_BWD_(F32, 8, 2, 4), DRIFT_FWD_(F32, 4, 4, 4),
+    DRIFT_BWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 1, 4),
     // short rows: several rows per wave
     GROUP_(F32, 4),
     // short rows that are not whole slots, dense: the tensor as one flat array
@@ -423,7 +424,15 @@ int drift_slots_for(const Problem& q, int fv) {
   if (half && (q.is_bwd || q.numseq > 2)) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
   if (q.numseq > q.at(2048)) return 0;
-  if (q.is_bwd && q.numseq * 16 >= q.cus && (q.numseq < q.at(128) || q.seqlen > 131072)) return 0;
+  // The backward of 16 to 127 rows with little work in all, and of more than 128 rows longer than 131072
+  // elements, stays with the sweep kernels' tiles of 16384 elements (24 x 262144 25.3 against 26.3 us, 40 x 196608
+  // 27.0 against 30.8 us, 512 x 262144 449.7 us with such tiles against 469.4 us; but 100 x 131072 55.1 against
+  // 48.5 us, 16 x 1048576 63.5 against 61.9 us, 32 x 1048576 123.1 against 118.0 us, 48 x 1048576 184.7 against
+  // 178.4 us, 64 x 524288 118.3 against 116.3 us, 128 x 262144 119.6 against 116.3 us).
+  if (q.is_bwd && q.numseq * 16 >= q.cus) {
+    if (q.numseq < q.at(128) && q.numseq * q.seqlen < 6 * 8192 * q.cus) return 0;
+    if (q.numseq > q.at(128) && q.seqlen > 131072) return 0;
+  }
   if (little_work_in_many_rows(q)) return 0;
   for (int s : {4, 2, 1}) {
     if (half != (s == 1)) continue;
@@ -867,9 +876,17 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     const bool drift = family == LINREC_FAMILY_DRIFT;
     if (q.elem_stride != 1 && q.seqlen != 1) return LINREC_E_UNSUPPORTED;
     if (q.numseq > 1 && q.row_stride < q.seqlen && q.row_stride > -q.seqlen) return LINREC_E_INVALID;
-    const int waves = tune && tune->waves > 0 ? tune->waves : 8;
+    int waves = tune && tune->waves > 0 ? tune->waves : 8;
     const int auto_slots = tune && tune->family != LINREC_FAMILY_AUTO ? 0 : drift ? drift_slots_for(q, fv) : sweep_slots_for(q, fv);
-    const int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? (drift ? 1 : 2) : 4);
+    int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? (drift ? 1 : 2) : 4);
+    // fp32 drift tiles of 4096 elements (every backward, and the forward of rows that are not whole tiles of
+    // 8192): 16 waves with one slot each rather than 8 waves with two.  Forward / backward in us: 512 x 65536
+    // backward 116.2 against 117.4, 300 x 65536 70.7 against 71.5, 1024 x 65536 229.2 against 231.2, 16 x 1048576
+    // 61.9 against 64.2, 1 x 33554432 74.6 / 119.8 against 82.1 / 125.0.
+    if (drift && !half && auto_slots == 2 && !(tune && (tune->waves > 0 || tune->slots > 0))) {
+      waves = 16;
+      slots = 1;
+    }
     const int64_t tile_elems = int64_t(waves) * slots * 64 * fv;
     // every tile of every row has to be a full one
     if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.seqlen % tile_elems != 0) return LINREC_E_UNSUPPORTED;

@@ -87,12 +87,12 @@ def _tunings_for(nat, L):
             out.append(nat.Tuning(nat.FAMILY_SWEEP, waves, slots, 3, 0))       # three teams share the rows
             if k % 2 == 0:
                 out.append(nat.Tuning(nat.FAMILY_SWEEP, waves, slots, 2, k // 2))  # two tiles of a row per walker
-    # the same launch shape with tiles stored two steps late (the backward is compiled for 8 waves x 2 slots only)
-    for waves, slots in [(8, 2), (8, 4), (4, 4)]:
+    # the same launch shape with tiles stored two steps late (the backward is compiled for tiles of 4096 elements only)
+    for waves, slots in [(8, 2), (8, 4), (4, 4), (16, 1)]:
         tile = waves * slots * 256
         if L % tile == 0 and L // tile <= 64:
             k = L // tile
-            both = (waves, slots) == (8, 2)
+            both = (waves, slots) in ((8, 2), (16, 1))
             out.append((nat.Tuning(nat.FAMILY_DRIFT, waves, slots, -1, 0), both))    # team = tiles of a row
             out.append((nat.Tuning(nat.FAMILY_DRIFT, waves, slots, 3, 0), both))     # three teams share the rows
             out.append((nat.Tuning(nat.FAMILY_DRIFT, waves, slots, 1, 1), both))     # one walker takes whole rows
@@ -809,25 +809,27 @@ def test_workspace_survives_many_launches_and_other_shapes(nat):
 
 @pytest.mark.parametrize("reverse", [False, True])
 @pytest.mark.parametrize("rows,tiles,slots,team", [(1, 130, 2, 130), (3, 256, 2, 256), (2, 192, 4, 96), (5, 96, 4, 96),
-                                                   (1, 200, 4, 200), (7, 65, 2, 65), (3, 512, 4, 0), (1, 1024, 4, 0)])
+                                                   (1, 200, 4, 200), (7, 65, 2, 65), (3, 512, 4, 0), (1, 1024, 4, 0),
+                                                   (1, 130, 1, 130), (3, 256, 1, 256), (2, 240, 1, 240), (7, 65, 1, 65)])
 def test_drift_teams_of_more_than_one_collecting_wave(nat, rows, tiles, slots, team, reverse):
     """Teams of more than 64 workgroups: every wave of a workgroup collects up to 64 of the team mates' maps
     and the waves' shares are composed after the barrier.  Forced team sizes on a few long rows (rows of
-    `tiles` tiles of 8 waves x `slots` slots), and the planner's own choice (team 0), which for so few rows
-    is one team of the whole chip.  The backward is compiled for 2 slots per lane."""
-    L = tiles * 8 * slots * 256
+    `tiles` tiles of 8 waves x `slots` slots, or of 16 waves x 1 slot), and the planner's own choice (team 0),
+    which for so few rows is one team of the whole chip.  The backward is compiled for tiles of 4096 elements."""
+    waves = 16 if slots == 1 else 8
+    L = tiles * waves * slots * 256
     x, c, dy = make_inputs((rows, L), "near1", seed=rows * 1000 + tiles)
-    tuning = nat.Tuning(nat.FAMILY_DRIFT, 8, slots, -1, team) if team else None
+    tuning = nat.Tuning(nat.FAMILY_DRIFT, waves, slots, -1, team) if team else None
     plan = nat.plan(x, reverse, False, tuning)
     assert plan["family"] == nat.FAMILY_DRIFT and plan["tasks"] == (team or 256) and plan["tasks"] > 64, plan
     label = f"drift {rows} x {tiles} tiles, team {plan['tasks']}"
-    if slots == 2 or tuning is None:
+    if slots <= 2 or tuning is None:
         _run_both(nat, x, c, dy, reverse, tuning, label)
     else:
         _run_forward(nat, x, c, reverse, tuning, label)
 
 
-@pytest.mark.parametrize("kind", ["look-back", "chain", "team", "sweep", "drift", "drift-200"])
+@pytest.mark.parametrize("kind", ["look-back", "chain", "team", "sweep", "drift", "drift-200", "drift-16-waves"])
 def test_tiny_poll_limit_ends_in_right_results_not_a_hang(nat, kind):
     """Failure handling, forced from the host: with a poll limit of one, a tile whose predecessors
     have not published by its second look gives up waiting and computes the value that enters it from
@@ -843,7 +845,8 @@ def test_tiny_poll_limit_ends_in_right_results_not_a_hang(nat, kind):
     tune = {"look-back": nat.Tuning(nat.FAMILY_TILE, 4, 4, 1), "chain": nat.Tuning(nat.FAMILY_TILE, 4, 4, 1, 2),
             "team": nat.Tuning(nat.FAMILY_TEAM, 8, 4, -1, 4), "sweep": nat.Tuning(nat.FAMILY_SWEEP, 8, 4, -1, 0),
             "drift": nat.Tuning(nat.FAMILY_DRIFT, 8, 2, -1, 0),            # the planner's teams of 120: two collecting waves
-            "drift-200": nat.Tuning(nat.FAMILY_DRIFT, 8, 2, -1, 200)}[kind]  # four collecting waves
+            "drift-200": nat.Tuning(nat.FAMILY_DRIFT, 8, 2, -1, 200),       # four collecting waves
+            "drift-16-waves": nat.Tuning(nat.FAMILY_DRIFT, 16, 1, -1, 200)}[kind]
     stream = torch.cuda.current_stream().cuda_stream
     want = oracle.fwd(x.cpu().numpy(), c.cpu().numpy(), False, dtype=np.float64)
     old = lib.linrec_set_spin_limit(1)

@@ -57,8 +57,8 @@ def test_planner_follows_the_compute_unit_count():
                 if cus == 20 and is_bwd:  # 16 rows are "many" for 20 CUs: one workgroup per row, nobody waits
                     assert p["family"] == nat.FAMILY_STREAM and p["workspace_bytes"] == 0
                     continue
-                # forward: teams whose tiles are stored two steps late; backward: teams that wait (tiles of 16384)
-                assert p["family"] == (nat.FAMILY_SWEEP if is_bwd else nat.FAMILY_DRIFT)
+                # teams whose tiles are stored two steps late
+                assert p["family"] == nat.FAMILY_DRIFT
                 # one workgroup per CU at most; whole teams only
                 assert p["grid"] <= cus and p["grid"] % p["tasks"] == 0
                 seen[(cus, is_bwd)] = p["grid"]
@@ -146,16 +146,16 @@ class TestPlanner:
         p2 = _plan((512, 65536))  # teams of 8 workgroups per row of 8 tiles, 32 teams, a tile stored two steps late
         assert p2["family"] == nat.FAMILY_DRIFT and (p2["slots"], p2["tasks"], p2["grid"], p2["tiles_per_row"]) == (4, 8, 256, 8)
         assert "drift_w8_s4_MODE_FWD_0" == names[p2["kernel_id"]] and p2["workspace_bytes"] > 0
-        p2b = _plan((512, 65536), is_bwd=True)  # the backward holds three tensors: tiles of 4096 elements
-        assert p2b["family"] == nat.FAMILY_DRIFT and (p2b["slots"], p2b["tasks"], p2b["grid"], p2b["tiles_per_row"]) == (2, 16, 256, 16)
-        assert "drift_w8_s2_MODE_BWD_1" == names[p2b["kernel_id"]]
+        p2b = _plan((512, 65536), is_bwd=True)  # the backward holds three tensors: tiles of 4096 elements, a slot for each of 16 waves
+        assert p2b["family"] == nat.FAMILY_DRIFT and (p2b["waves"], p2b["slots"], p2b["tasks"], p2b["grid"], p2b["tiles_per_row"]) == (16, 1, 16, 256, 16)
+        assert "drift_w16_s1_MODE_BWD_1" == names[p2b["kernel_id"]] and p2b["block"] == 1024
         p3 = _plan((16384, 2048), reverse=True)
         assert (p3["waves"], p3["slots"], p3["carry"]) == (4, 2, 0) and "FWD_1" in names[p3["kernel_id"]]
         p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 128 (a whole row in flight each) that go from row to row
         assert p4["family"] == nat.FAMILY_DRIFT and p4["carry"] == 1 and p4["workspace_bytes"] > 0
         assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (128, 256, 128)
-        p4bw = _plan((16, 1048576), is_bwd=True)  # the backward takes tiles of 16384 elements
-        assert (p4bw["family"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_SWEEP, 8, 16, 256, 64)
+        p4bw = _plan((16, 1048576), is_bwd=True)  # the backward: one team of the whole launch, tiles of 4096 elements
+        assert (p4bw["family"], p4bw["waves"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_DRIFT, 16, 1, 256, 256, 256)
         p4r = _plan((16, 1048576 + 4))  # a ragged last tile: one team per row
         assert p4r["family"] == nat.FAMILY_TEAM and p4r["grid"] == 16 * p4r["tasks"] and 2 <= p4r["tasks"] <= 64
         for rows, is_bwd in ((1, False), (2, False), (3, True), (6, True)):
@@ -229,7 +229,10 @@ class TestPlanner:
             assert fam(shape, True) == D, shape
         # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup each
         assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST] * 6
-        assert fam((96, 65536), True) == W and fam((16, 1 << 20), True) == W and fam((512, 262144), True) == W
+        # the backward of 16 to 127 rows with little work in all, and of more than 128 rows longer than 131072
+        # elements: teams that wait, with tiles of 16384 elements
+        assert fam((96, 65536), True) == W and fam((24, 262144), True) == W and fam((512, 262144), True) == W
+        assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
         # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
         assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
@@ -268,12 +271,12 @@ class TestPlanner:
         hb = lambda n: fam((n, 262144), True, dtype=torch.bfloat16)
         assert [hb(n) for n in (32, 48, 64, 80, 128)] == [nat.FAMILY_TEAM] * 5
         assert [hb(n) for n in (96, 100, 160)] == [nat.FAMILY_SWEEP] * 3
-        assert fam((64, 262144), dtype=torch.float16) == nat.FAMILY_SWEEP and fam((64, 262144), True) == nat.FAMILY_SWEEP
+        assert fam((64, 262144), dtype=torch.float16) == nat.FAMILY_SWEEP and fam((64, 262144), True) == D
         pf, pb = nat.plan(torch.empty(300, 65536)), nat.plan(torch.empty(300, 65536), False, True)
         assert (pf["tasks"], pf["grid"]) == (8, 256) and (pb["tasks"], pb["grid"]) == (16, 256)
         p = nat.plan(torch.empty(40, 8192 * 24))                    # 24 tiles: teams of 24, 10 of them
         p2 = nat.plan(torch.empty(300, 4096 * 9))                   # whole tiles of 4096 elements only
-        assert (p2["family"], p2["slots"], p2["tasks"], p2["tiles_per_row"], p2["grid"]) == (D, 2, 9, 9, 252)
+        assert (p2["family"], p2["waves"], p2["slots"], p2["tasks"], p2["tiles_per_row"], p2["grid"]) == (D, 16, 1, 9, 9, 252)
         assert p["family"] == D and (p["tasks"], p["grid"]) == (24, 240)
         p = nat.plan(torch.empty(40, 8192 * 24), False, True)       # the backward of 16 to 127 rows waits
         assert p["family"] == W and p["tasks"] == 12
