@@ -34,8 +34,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("C1", "tile_w8_s2_v4_MODE_FWD_0_0"): 3.195e6,
     ("C1", "tile_w8_s2_v4_MODE_BWD_1_0"): 5.362e6,
     ("C2", "drift_w8_s4_MODE_FWD_0"): 403.83e6,
+    ("C2", "drift_w16_s2_MODE_FWD_0"): 403.68e6,
     ("C2", "drift_w8_s2_MODE_BWD_1"): 674.74e6,
-    ("C2", "drift_w16_s1_MODE_BWD_1"): 674.78e6,
+    ("C2", "drift_w16_s1_MODE_BWD_1"): 674.87e6,
     ("C2", "stream_w8_s4_MODE_FWD_0"): 402.71e6,
     ("C2", "stream_w8_s4_MODE_BWD_1"): 671.42e6,
     ("C2", "sweep_w8_s4_MODE_BWD_1"): 673.19e6,

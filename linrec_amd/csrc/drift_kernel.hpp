@@ -38,8 +38,9 @@ namespace linrec {
 //
 // The loop is unrolled three steps deep so that the three tiles in the works (being scanned, and stored
 // one and two steps from now) and the tiles of loaded data change roles without a register being copied.
-// PF: tiles of loads in flight ahead of the scan (1 or 2); WPE: waves per SIMD the compiler is to allow for.
-template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1>
+// PF: tiles of loads in flight ahead of the scan (1 or 2); WPE: waves per SIMD the compiler is to allow for;
+// WIDE: teams of more than 64 are served (the forward with 16 waves of two slots has no registers for that).
+template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1, bool WIDE = true>
 __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   static_assert(PF == 1 || PF == 2, "one or two tiles of loads ahead of the scan");
   static_assert(NW <= 16, "the waves' shares are composed inside a DPP row");
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   // A team of at most 64: wave 0 holds all the maps and has the value entering the tile in LDS before the
   // barrier; the others only read it afterwards.  Larger teams: every wave leaves its share in LDS before
   // the barrier and composes all the shares for itself after it.
-  const bool wide = M > 64;
+  const bool wide = WIDE && M > 64;
   // Before the barrier: the words asked for (asked for again while a team mate is more than two steps
   // behind) composed, oldest first.  A wait that runs out: wave 0 of a team of at most 64 computes the
   // value from the row's own data on the spot; in a larger team the wave notes it in LDS and the workgroup
@@ -252,6 +253,20 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     }
     Pending& now = P[PH];
     tile_scan<S, VEC, MODE>(d, now.r);
+    if constexpr (MODE == MODE_FWD) {
+      // a slot's map from the wave's entry value to the slot's is folded into the elements' maps, which leaves
+      // a pending tile two values per element and nothing per slot (16 waves have 128 registers each)
+#pragma unroll
+      for (int j = 0; j < S; ++j) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
+          now.r.pa[j][i] *= now.r.ex_a[j];
+        }
+        now.r.ex_a[j] = 1.0f;
+        now.r.ex_b[j] = 0.0f;
+      }
+    }
     const int par = n & 1;
     if (lane == 0) {
       sh_a[par][wave] = now.r.total.a;

@@ -79,7 +79,7 @@ struct KernelEntry {
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, ((NW) > 8 ? 4 : 2)>, DT, LINREC_FAMILY_DRIFT, \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
@@ -205,9 +205,8 @@ const KernelEntry kKernels[] = {
     SWEEP_(F32, 8, 4, 4), SWEEP_(F32, 8, 2, 4), SWEEP_(F32, 4, 4, 4), SWEEP_(F32, 8, 8, 4),
     // the same launch shape with a tile stored two steps late, so that nobody waits for the exchange
     DRIFT_FWD_(F32, 8, 4, 4), DRIFT_FWD_(F32, 8, 2, 4), DRIFT_BWD_(F32, 8, 2, 4), DRIFT_FWD_(F32, 4, 4, 4),
-    // (16 waves of two slots forward need 140 registers where 128 are to be had: 60 bytes of scratch per lane and
-    // 512 x 65536 72.7 against 68.2 us for 8 waves of four slots)
-    DRIFT_BWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 1, 4),
+    // (16 waves of two slots forward: the 128 registers to be had suffice for teams of at most 64)
+    DRIFT_BWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 2, 4),
     // short rows: several rows per wave
     GROUP_(F32, 4),
     // short rows that are not whole slots, dense: the tensor as one flat array
@@ -414,6 +413,9 @@ int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int6
 bool little_work_in_many_rows(const Problem& q) {
   return q.dtype == LINREC_DTYPE_F32 && q.numseq * 4 >= q.cus && q.numseq * q.seqlen <= 4 * 8192 * q.cus;
 }
+// The largest team a drift kernel of this geometry serves: a lane of a wave per team mate, in every wave - except
+// 16 waves of two slots, compiled for one collecting wave.
+int64_t drift_max_team(int waves, int slots) { return waves == 16 && slots == 2 ? 64 : int64_t(64) * waves; }
 // Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
 int drift_slots_for(const Problem& q, int fv) {
   // 16-bit storage: one kernel, forward, tiles of 4096 elements (more per lane do not fit the registers, nor
@@ -889,6 +891,15 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       waves = 16;
       slots = 1;
     }
+    // The forward's tiles of 8192 elements likewise, 16 waves of two slots rather than 8 of four, in teams of at
+    // most 64 (one after the other in one process, us: 512 x 65536 67.9 against 68.5, 300 x 65536 42.3 against
+    // 43.6, 1024 x 65536 132.2 against 133.8, 16 x 1048576 in teams of 128 37.6 against 38.1 - compiled without
+    // the larger teams' code, which does not fit its registers, so those keep 8 waves).
+    if (drift && !half && !q.is_bwd && auto_slots == 4 && !(tune && (tune->waves > 0 || tune->slots > 0)) &&
+        drift_team_size(q, q.seqlen / (int64_t(8) * 4 * 64 * fv), 8, q.cus) <= 64) {
+      waves = 16;
+      slots = 2;
+    }
     const int64_t tile_elems = int64_t(waves) * slots * 64 * fv;
     // every tile of every row has to be a full one
     if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.seqlen % tile_elems != 0) return LINREC_E_UNSUPPORTED;
@@ -903,7 +914,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
                              ? tune->tasks
                              : drift ? drift_team_size(q, tiles_per_row, waves, resident)
                                      : sweep_team_size(tiles_per_row, std::min<int64_t>(kSweepMaxTeam, resident));
-    if (team > (drift ? 64 * waves : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
+    if (team > (drift ? drift_max_team(waves, slots) : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
     int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
     if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;
@@ -1257,6 +1268,8 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
       a.ws_tiles = lay.tiles;
     }
     a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+    // (a plan made elsewhere, or edited: never a team the kernel was not compiled for)
+    if (plan.family == LINREC_FAMILY_DRIFT && a.tasks > drift_max_team(k.waves, k.slots)) return LINREC_E_INVALID;
 #ifdef LINREC_PHASE_TIMING
     a.timing = g_timing_buffer;
 #endif

@@ -88,7 +88,7 @@ def _tunings_for(nat, L):
             if k % 2 == 0:
                 out.append(nat.Tuning(nat.FAMILY_SWEEP, waves, slots, 2, k // 2))  # two tiles of a row per walker
     # the same launch shape with tiles stored two steps late (the backward is compiled for tiles of 4096 elements only)
-    for waves, slots in [(8, 2), (8, 4), (4, 4), (16, 1)]:
+    for waves, slots in [(8, 2), (8, 4), (4, 4), (16, 1), (16, 2)]:
         tile = waves * slots * 256
         if L % tile == 0 and L // tile <= 64:
             k = L // tile

@@ -144,8 +144,8 @@ class TestPlanner:
         p1 = _plan((64, 4096))
         assert p1["family"] == nat.FAMILY_TILE and p1["carry"] == 0 and p1["grid"] == 64
         p2 = _plan((512, 65536))  # teams of 8 workgroups per row of 8 tiles, 32 teams, a tile stored two steps late
-        assert p2["family"] == nat.FAMILY_DRIFT and (p2["slots"], p2["tasks"], p2["grid"], p2["tiles_per_row"]) == (4, 8, 256, 8)
-        assert "drift_w8_s4_MODE_FWD_0" == names[p2["kernel_id"]] and p2["workspace_bytes"] > 0
+        assert p2["family"] == nat.FAMILY_DRIFT and (p2["waves"], p2["slots"], p2["tasks"], p2["grid"], p2["tiles_per_row"]) == (16, 2, 8, 256, 8)
+        assert "drift_w16_s2_MODE_FWD_0" == names[p2["kernel_id"]] and p2["workspace_bytes"] > 0
         p2b = _plan((512, 65536), is_bwd=True)  # the backward holds three tensors: tiles of 4096 elements, a slot for each of 16 waves
         assert p2b["family"] == nat.FAMILY_DRIFT and (p2b["waves"], p2b["slots"], p2b["tasks"], p2b["grid"], p2b["tiles_per_row"]) == (16, 1, 16, 256, 16)
         assert "drift_w16_s1_MODE_BWD_1" == names[p2b["kernel_id"]] and p2b["block"] == 1024
@@ -153,6 +153,10 @@ class TestPlanner:
         assert (p3["waves"], p3["slots"], p3["carry"]) == (4, 2, 0) and "FWD_1" in names[p3["kernel_id"]]
         p4 = _plan((16, 1048576))  # rows of whole tiles: teams of 128 (a whole row in flight each) that go from row to row
         assert p4["family"] == nat.FAMILY_DRIFT and p4["carry"] == 1 and p4["workspace_bytes"] > 0
+        assert (p4["waves"], p4["slots"]) == (8, 4)  # (teams of more than 64: the kernel of 8 waves)
+        with pytest.raises(NotImplementedError):     # 16 waves of two slots are compiled for teams of at most 64
+            _plan((16, 1048576), tuning=nat.Tuning(nat.FAMILY_DRIFT, 16, 2, -1, 128))
+        assert _plan((16, 1048576), tuning=nat.Tuning(nat.FAMILY_DRIFT, 16, 2, -1, 64))["tasks"] == 64
         assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (128, 256, 128)
         p4bw = _plan((16, 1048576), is_bwd=True)  # the backward: one team of the whole launch, tiles of 4096 elements
         assert (p4bw["family"], p4bw["waves"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_DRIFT, 16, 1, 256, 256, 256)
