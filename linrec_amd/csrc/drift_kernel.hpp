@@ -255,13 +255,15 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     tile_scan<S, VEC, MODE>(d, now.r);
     if constexpr (MODE == MODE_FWD) {
       // a slot's map from the wave's entry value to the slot's is folded into the elements' maps, which leaves
-      // a pending tile two values per element and nothing per slot (16 waves have 128 registers each)
+      // a pending tile two values per element and nothing per slot (16 waves have 128 registers each); nothing
+      // enters a row's first wave, whose factors are therefore zero and never meet a product that overflowed
+      const bool nothing_enters = it.t == 0 && wave == 0;
 #pragma unroll
       for (int j = 0; j < S; ++j) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
           now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
-          now.r.pa[j][i] *= now.r.ex_a[j];
+          now.r.pa[j][i] = nothing_enters ? 0.0f : now.r.pa[j][i] * now.r.ex_a[j];
         }
         now.r.ex_a[j] = 1.0f;
         now.r.ex_b[j] = 0.0f;
