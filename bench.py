@@ -34,9 +34,9 @@ MEASURED_TRAFFIC_BYTES = {
     ("C1", "tile_w8_s2_v4_MODE_FWD_0_0"): 3.195e6,
     ("C1", "tile_w8_s2_v4_MODE_BWD_1_0"): 5.362e6,
     ("C2", "drift_w8_s4_MODE_FWD_0"): 403.83e6,
-    ("C2", "drift_w16_s2_MODE_FWD_0"): 403.68e6,
+    ("C2", "drift_w16_s2_MODE_FWD_0"): 403.67e6,
     ("C2", "drift_w8_s2_MODE_BWD_1"): 674.74e6,
-    ("C2", "drift_w16_s1_MODE_BWD_1"): 674.87e6,
+    ("C2", "drift_w16_s1_MODE_BWD_1"): 674.64e6,
     ("C2", "stream_w8_s4_MODE_FWD_0"): 402.71e6,
     ("C2", "stream_w8_s4_MODE_BWD_1"): 671.42e6,
     ("C2", "sweep_w8_s4_MODE_BWD_1"): 673.19e6,
@@ -45,7 +45,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("C4", "drift_w8_s4_MODE_FWD_0"): 202.32e6,
     ("C4", "sweep_w8_s4_MODE_FWD_0"): 202.13e6,
     ("C4", "sweep_w8_s8_MODE_BWD_1"): 336.69e6,
-    ("C4", "drift_w16_s1_MODE_BWD_1"): 337.57e6,
+    ("C4", "drift_w16_s1_MODE_BWD_1"): 337.58e6,
     ("C5", "column_v2_u8_MODE_FWD_0"): 805.12e6,
     ("C5", "column_v2_u8_MODE_BWD_1"): 1340.78e6,
     ("C2", "bf16_stream_w8_s2_MODE_FWD_0"): 201.40e6,

@@ -77,9 +77,14 @@ struct KernelEntry {
 #define SWEEP_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
   SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
+// Tiles of loads in flight ahead of the scan: two in the backward with 16 waves of one slot, whose step loads
+// only 48 KB (one after the other in one process, us, against 8 waves of two slots with one tile ahead, which one
+// tile ahead in 16 waves had beaten by 1 to 4 %: 512 x 65536 112.4 against 117.5, 300 x 65536 68.3 against 71.2,
+// 16 x 1048576 60.1 against 63.6, 1 x 33554432 111.6 against 124.5); the forward gains nothing from it.
+#define DRIFT_TILES_AHEAD(NW, S, MODE) ((NW) == 16 && (S) == 1 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, 1, ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
@@ -428,15 +433,12 @@ int drift_slots_for(const Problem& q, int fv) {
   if (half && (q.is_bwd || q.numseq > 2)) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
   if (q.numseq > q.at(2048)) return 0;
-  // The backward of 16 to 127 rows with little work in all, and of more than 128 rows longer than 131072
-  // elements, stays with the sweep kernels' tiles of 16384 elements (24 x 262144 25.3 against 26.3 us, 40 x 196608
-  // 27.0 against 30.8 us, 512 x 262144 449.7 us with such tiles against 469.4 us; but 100 x 131072 55.1 against
-  // 48.5 us, 16 x 1048576 63.5 against 61.9 us, 32 x 1048576 123.1 against 118.0 us, 48 x 1048576 184.7 against
-  // 178.4 us, 64 x 524288 118.3 against 116.3 us, 128 x 262144 119.6 against 116.3 us).
-  if (q.is_bwd && q.numseq * 16 >= q.cus) {
-    if (q.numseq < q.at(128) && q.numseq * q.seqlen < 6 * 8192 * q.cus) return 0;
-    if (q.numseq > q.at(128) && q.seqlen > 131072) return 0;
-  }
+  // The backward of 16 to 127 rows with little work in all stays with the sweep kernels' tiles of 16384 elements
+  // (24 x 262144 25.3 against 26.3 us, 40 x 196608 27.0 against 30.8 us; but 100 x 131072 55.1 against 48.5 us,
+  // 16 x 1048576 63.5 against 61.9 us, 32 x 1048576 123.1 against 118.0 us, 64 x 524288 118.3 against 116.3 us -
+  // all with one tile of loads ahead; with two, 64 x 524288 takes 112.6 us, 256 x 262144 219.7 against 232.8 us and
+  // 512 x 262144 453.1 against 452.3 us).
+  if (q.is_bwd && q.numseq * 16 >= q.cus && q.numseq < q.at(128) && q.numseq * q.seqlen < 6 * 8192 * q.cus) return 0;
   if (little_work_in_many_rows(q)) return 0;
   for (int s : {4, 2, 1}) {
     if (half != (s == 1)) continue;

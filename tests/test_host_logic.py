@@ -54,9 +54,6 @@ def test_planner_follows_the_compute_unit_count():
             assert lib.linrec_compute_units() == cus
             for is_bwd in (False, True):
                 p = nat.plan(x, False, is_bwd)
-                if cus == 20 and is_bwd:  # 16 rows are "many" for 20 CUs: one workgroup per row, nobody waits
-                    assert p["family"] == nat.FAMILY_STREAM and p["workspace_bytes"] == 0
-                    continue
                 # teams whose tiles are stored two steps late
                 assert p["family"] == nat.FAMILY_DRIFT
                 # one workgroup per CU at most; whole teams only
@@ -233,10 +230,10 @@ class TestPlanner:
             assert fam(shape, True) == D, shape
         # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup each
         assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST] * 6
-        # the backward of 16 to 127 rows with little work in all, and of more than 128 rows longer than 131072
-        # elements: teams that wait, with tiles of 16384 elements
-        assert fam((96, 65536), True) == W and fam((24, 262144), True) == W and fam((512, 262144), True) == W
+        # the backward of 16 to 127 rows with little work in all: teams that wait, with tiles of 16384 elements
+        assert fam((96, 65536), True) == W and fam((24, 262144), True) == W
         assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
+        assert fam((512, 262144), True) == D and fam((256, 262144), True) == D
         # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
         assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
