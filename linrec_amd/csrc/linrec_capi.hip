@@ -421,7 +421,8 @@ bool little_work_in_many_rows(const Problem& q) {
 // The largest team a drift kernel of this geometry serves: a lane of a wave per team mate, in every wave - except
 // 16 waves of two slots, compiled for one collecting wave.
 int64_t drift_max_team(int waves, int slots) { return waves == 16 && slots == 2 ? 64 : int64_t(64) * waves; }
-// Returns the slots per lane to use (tiles of 8 waves), 0 for "not a drift case".
+// Returns the tile to use as slots per lane of 8 waves (4: 8192 fp32 elements, 2: 4096), 0 for "not a drift
+// case"; which kernel serves the tile (8 waves, or 16 with half the slots) is the launch planner's business.
 int drift_slots_for(const Problem& q, int fv) {
   // 16-bit storage: one kernel, forward, tiles of 4096 elements (more per lane do not fit the registers, nor
   // does any backward).  A step of so little data costs more than the exchange it hides wherever other
