@@ -395,8 +395,8 @@ int64_t sweep_team_size(int64_t tiles_per_row, int64_t most = kSweepMaxTeam) {
 // more of a row is in flight at once, the fewer gaps the launch's reading positions leave.  A lane of a
 // wave per team mate: at most 64 a wave.
 int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int64_t resident) {
-  int64_t best = 1;
-  double best_busy = 0.0;
+  int64_t best = 1, best_large = 0;
+  double best_busy = 0.0, best_large_busy = 0.0;
   for (int64_t team = std::min<int64_t>({int64_t(64) * waves, resident, tiles_per_row}); team >= 1; --team) {
     if (tiles_per_row % team != 0) continue;
     const int64_t teams = std::min(q.numseq, resident / team);
@@ -406,8 +406,13 @@ int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int6
       best = team;
       best_busy = busy;
     }
+    if (team >= kSweepMinTiles && busy > best_large_busy + 1e-9) {
+      best_large = team;
+      best_large_busy = busy;
+    }
   }
-  return best;
+  // (a team too small to be worth the exchange only where no larger one keeps the chip nearly as busy)
+  return best < kSweepMinTiles && best_large_busy >= 0.95 * best_busy ? best_large : best;
 }
 // Many rows with little work for each workgroup (at most four tiles of 8192 elements for each compute unit):
 // filling and draining the three tiles a drift kernel has in the works costs more than the exchange it saves,
@@ -433,7 +438,13 @@ int drift_slots_for(const Problem& q, int fv) {
   const bool half = q.dtype != LINREC_DTYPE_F32;
   if (half && (q.is_bwd || q.numseq > 2)) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
-  if (q.numseq > q.at(2048)) return 0;
+  // More than 2048 rows: the forward only, in tiles of 4096 elements (16 waves of one slot).  Forward / backward in
+  // us against one workgroup per row forward and the sweep kernels backward: 4096 x 32768 261.7 / 453.2 against
+  // 279.8 / 470.4, 8192 x 32768 543.5 / 965.4 against 565.3 / 964.1, 3000 x 65536 389.9 / 672.2 against 395.8 / 659.5,
+  // 4096 x 65536 532.2 / 948.0 against 543.9 / 934.5 (tiles of 8192 in 16 waves of two slots: 271.0, 569.5, 391.9,
+  // 540.6 forward).
+  const bool many_rows = q.numseq > q.at(2048);
+  if (many_rows && q.is_bwd) return 0;
   // The backward of 16 to 127 rows with little work in all stays with the sweep kernels' tiles of 16384 elements
   // (24 x 262144 25.3 against 26.3 us, 40 x 196608 27.0 against 30.8 us; but 100 x 131072 55.1 against 48.5 us,
   // 16 x 1048576 63.5 against 61.9 us, 32 x 1048576 123.1 against 118.0 us, 64 x 524288 118.3 against 116.3 us -
@@ -444,11 +455,14 @@ int drift_slots_for(const Problem& q, int fv) {
   for (int s : {4, 2, 1}) {
     if (half != (s == 1)) continue;
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
+    if (many_rows && s == 4) continue;
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
     const int64_t tiles_per_row = q.seqlen / tile;
     const int64_t team = drift_team_size(q, tiles_per_row, 8, q.cus);
     if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
+    // (a caller that can only give so much workspace is served by the kernels that need less)
+    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
     // fp32 rows of fewer than eight tiles of 4096 elements: one workgroup per row does as well or better
     // (forward / backward in us: 768 x 16384 27.3 / 46.3 against 32.3 / 47.5, 400 x 24576 22.6 / 36.4 against
     // 26.3 / 39.7, 1000 x 24576 52.2 / 89.3 against 55.7 / 90.3, 1536 x 16384 52.4 / 90.4 against 55.3 / 89.7,

@@ -659,6 +659,29 @@ def test_little_work_in_many_rows_goes_to_small_teams_with_the_largest_tiles(nat
 
 
 @pytest.mark.parametrize("reverse", [False, True])
+def test_more_than_2048_rows_of_whole_tiles_run_forward_in_teams(nat, reverse):
+    """Beyond 2048 rows the forward still goes to the teams whose tiles are stored two steps late (tiles of 4096
+    elements, 16 waves), the backward to the teams that wait or to one workgroup per row."""
+    dev = torch.device("cuda:0")
+    for n, L, team in [(2100, 32768, 8), (2200, 4096 * 9, 9)]:
+        g = torch.Generator().manual_seed(n)
+        x, c, dy = (torch.randn(n, L, generator=g), torch.rand(n, L, generator=g), torch.randn(n, L, generator=g))
+        xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+        plan = nat.plan(xd, reverse)
+        assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == (nat.FAMILY_DRIFT, 16, 1, team), plan
+        assert nat.plan(xd, reverse, True)["family"] in (nat.FAMILY_SWEEP, nat.FAMILY_STREAM)
+        y = nat.fwd(xd, cd, reverse)
+        dx, dc = nat.bwd(dyd, cd, y, reverse)
+        torch.cuda.synchronize()
+        y_t, _, _ = truth(x, c, dy, reverse)
+        dx_t, dc_t = oracle.bwd(dy.numpy(), c.numpy(), y.cpu().numpy().astype(np.float64), reverse, dtype=np.float64)
+        check_close(y, y_t, f"{n} x {L} outputs")
+        check_close(dx, dx_t, f"{n} x {L} d_inputs")
+        check_close(dc, dc_t, f"{n} x {L} d_coeffs")
+    assert nat.gave_up_count() == 0
+
+
+@pytest.mark.parametrize("reverse", [False, True])
 def test_broadcast_inputs_get_dense_results(nat, reverse):
     """Expanded tensors (zero strides: a value per row repeated along the scan axis, a row repeated for
     every row, a scalar) are valid inputs; results must not inherit strides under which elements share

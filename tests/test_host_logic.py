@@ -234,12 +234,15 @@ class TestPlanner:
         assert fam((96, 65536), True) == W and fam((24, 262144), True) == W
         assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
         assert fam((512, 262144), True) == D and fam((256, 262144), True) == D
-        # more rows than that: one workgroup per row forward, teams that wait backward (up to 1024 rows of 16 tiles and more)
-        assert fam((4096, 65536)) == ST and fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST
+        # more than 2048 rows: the forward still, in tiles of 4096 elements; the backward in teams that wait (up to
+        # 1024 rows of 16 tiles and more) or one workgroup per row; ragged rows one workgroup per row
+        q = nat.plan(torch.empty(4096, 65536))
+        assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 16, 256), q
+        assert fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST and fam((4096, 65536 + 8)) == ST
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
         # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
-        assert slots((4096, 65536)) == 8 and slots((2304, 131072), True) == 8
+        assert slots((2304, 131072), True) == 8 and slots((256, 131072), True) == 1
         assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
@@ -460,7 +463,7 @@ class TestPlanner:
         assert lib.linrec_plan_f32(None, 4, 10, 5, 1, 0, 0, None, ctypes.byref(plan)) == -1  # rows overlap
         assert lib.linrec_plan_f32(None, 4, 2 ** 31, 2 ** 31, 1, 0, 0, None, ctypes.byref(plan)) == -4
         assert lib.linrec_workspace_bytes(16, 1 << 20, 1 << 20, 1, 0, 0, None) > 0
-        assert lib.linrec_workspace_bytes(4096, 65536, 65536, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
+        assert lib.linrec_workspace_bytes(4096, 65540, 65540, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
         assert lib.linrec_workspace_bytes_for_tiles(0) == 0
         assert lib.linrec_workspace_bytes_for_tiles(1000) >= 16 + 16 * 1000
 

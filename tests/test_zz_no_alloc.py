@@ -105,3 +105,24 @@ def test_noalloc_takes_another_kernel_where_the_usual_choice_needs_more_scratch_
     t = nat.Tuning(nat.FAMILY_COLDRIFT)
     assert lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0,
                                   ctypes.byref(t), torch.cuda.current_stream().cuda_stream) == -5
+
+
+def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row():
+    """20000 rows of 32768 elements: linrec_fwd takes teams that go from row to row, whose per-tile maps need more
+    than the 4 MiB there are; the entry point that allocates nothing walks every row with one workgroup instead."""
+    lib = nat.lib()
+    x, c = _pair((20000, 32768), 6)
+    lay = nat.row_layout(x)
+    need = lib.linrec_workspace_bytes_dtype(nat.DTYPES[x.dtype], *lay, 0, 0, None)
+    assert nat.plan(x)["family"] == nat.FAMILY_DRIFT and need > (4 << 20)
+    got = torch.full_like(x, float("nan"))
+    rc = lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0, None,
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    want = nat.fwd(x, c)
+    torch.cuda.synchronize()
+    assert not torch.isnan(got).any()
+    rows = torch.tensor([0, 1, 255, 256, 9999, 19999], device=x.device)
+    truth = oracle.fwd(x.index_select(0, rows).cpu().numpy(), c.index_select(0, rows).cpu().numpy(), False, dtype=np.float64)
+    assert oracle.error_report(got.index_select(0, rows).cpu().numpy(), truth)["normwise"] <= 1e-5
+    assert oracle.error_report(want.index_select(0, rows).cpu().numpy(), truth)["normwise"] <= 1e-5
