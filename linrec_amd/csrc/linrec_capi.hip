@@ -467,7 +467,9 @@ int drift_slots_for(const Problem& q, int fv) {
     // (forward / backward in us: 768 x 16384 27.3 / 46.3 against 32.3 / 47.5, 400 x 24576 22.6 / 36.4 against
     // 26.3 / 39.7, 1000 x 24576 52.2 / 89.3 against 55.7 / 90.3, 1536 x 16384 52.4 / 90.4 against 55.3 / 89.7,
     // 2048 x 16384 68.9 / 120.0 against 70.4 / 117.4)
-    if (s == 2 && tiles_per_row < 8) continue;
+    // (with 16 waves and two tiles of loads ahead the backward of 512 rows and more gains from four such tiles on:
+    // 2048 x 16384 111.8 against 119.0 us, 768 x 16384 43.9 against 45.5 us)
+    if (s == 2 && tiles_per_row < 8 && !(q.is_bwd && q.numseq >= q.at(512))) continue;
     // the teams have to fill at least half the chip, and every member gets a few tiles (1 x 4194304 in four
     // steps of 4096 elements: 16.4 / 19.8 us, what look-back tiles take)
     if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < (s == 4 ? 3 : 4) * q.cus) continue;

@@ -228,8 +228,9 @@ class TestPlanner:
         assert fam((130, 65536)) == D and fam((63, 131072)) == D and fam((128, 65536), dtype=torch.bfloat16) == W
         for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 32768)]:
             assert fam(shape, True) == D, shape
-        # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup each
-        assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST] * 6
+        # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup
+        # each, except the backward of 512 rows and more with at least four such tiles
+        assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST, D, ST, D, ST, ST]
         # the backward of 16 to 127 rows with little work in all: teams that wait, with tiles of 16384 elements
         assert fam((96, 65536), True) == W and fam((24, 262144), True) == W
         assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
