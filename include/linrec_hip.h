@@ -68,8 +68,10 @@ extern "C" {
 #define LINREC_FAMILY_DRIFT 10  /* the SWEEP launch shape with the exchange between team mates off the critical
                                   path: a scanned tile is kept in registers and stored two steps late, by which
                                   time the value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
-                                  teams of up to 64 a wave (512 for 8 waves): beyond 64 every wave collects maps.
-                                  fp32: 8 waves x 4 or 2 slots forward, 8 x 2 backward; 16-bit storage: 8 x 1, forward */
+                                  teams of up to 64 a wave: beyond 64 every wave collects maps.  Compiled (waves x slots):
+                                  fp32 forward 8 x 4, 8 x 2, 4 x 4, 16 x 1 and 16 x 2 (the last for teams of at most
+                                  64 only), fp32 backward 8 x 2 and 16 x 1; 16-bit storage 8 x 1, forward only.
+                                  The planner's picks are the 16-wave ones, and 8 x 4 forward for teams beyond 64 */
 
 #define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
                                    of workgroups share a block of rows and take its steps along the scan axis in
@@ -274,6 +276,17 @@ int linrec_plan_f32(const void* any_input, int64_t numseq, int64_t seqlen, int64
  * hipFuncGetAttributes' numRegs, sharedSizeBytes (LDS), localSizeBytes (scratch) and
  * maxThreadsPerBlock.
  */
+/*
+ * The planner's crossover thresholds between the long-row kernels, as compiled in from the generated
+ * table csrc/plan_thresholds.inc (written by `python -m linrec_amd.tune --write-table` from timings on the
+ * device).  The role of the dispatch table the reference's grid search writes (eval/tune.py:104-134);
+ * reading them back lets a harness or a test check what the planner decides by.
+ * name: NULL beyond the last index; value: -1 beyond the last index.
+ */
+int linrec_plan_threshold_count(void);
+const char* linrec_plan_threshold_name(int index);
+int64_t linrec_plan_threshold_value(int index);
+
 int linrec_kernel_count(void);
 const char* linrec_kernel_name(int kernel_id);
 int linrec_kernel_attrs(int kernel_id, int* num_regs, int* lds_bytes, int* scratch_bytes,

@@ -84,6 +84,9 @@ def _declare(lib):
         "linrec_compute_units": (i32, []),
         "linrec_set_compute_units": (i32, [i32]),
         "linrec_fwd_noalloc": (i32, [i32, p, p, p, i64, i64, i64, i64, i32, tun, p]),
+        "linrec_plan_threshold_count": (i32, []),
+        "linrec_plan_threshold_name": (ctypes.c_char_p, [i32]),
+        "linrec_plan_threshold_value": (i64, [i32]),
         "linrec_kernel_count": (i32, []),
         "linrec_kernel_name": (ctypes.c_char_p, [i32]),
         "linrec_kernel_attrs": (i32, [i32] + [ctypes.POINTER(ctypes.c_int)] * 4),
@@ -541,6 +544,13 @@ def kernel_table():
     """Names of all compiled kernels (role of _C.config_list, linrec/impl/cuda/extension.cpp:38-39)."""
     L = lib()
     return [L.linrec_kernel_name(i).decode() for i in range(L.linrec_kernel_count())]
+
+
+def plan_thresholds():
+    """{name: value} of the planner's generated crossover thresholds (csrc/plan_thresholds.inc as compiled in)."""
+    L = lib()
+    return {L.linrec_plan_threshold_name(i).decode(): int(L.linrec_plan_threshold_value(i))
+            for i in range(L.linrec_plan_threshold_count())}
 
 
 def kernel_attrs(kernel_id):

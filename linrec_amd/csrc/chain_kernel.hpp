@@ -39,7 +39,7 @@ __global__ __launch_bounds__(64 * NW) void chain_kernel(TileArgs p) {
 
   uint32_t seq = 0;
   uint32_t leaf_count = 0;
-  if (wave == 0) seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (wave == 0) seq = load_seq_through_caches(p.ws);
 
   const int u_wave = k * TILE_SLOTS + wave * WAVE_SLOTS;
   const bool row_start = k == 0 && wave == 0;

@@ -143,20 +143,27 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   auto collect = [&](int k, Words w, int slot, int token) {
     const int need = k < M - 1 ? k : M - 1;
     if (wave >= need) return;
-    for (int polls = 0;; ++polls) {
+    auto all_there = [&]() {
       bool have = true;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) have = have && uint32_t(w.w0[e] >> 32) == want && uint32_t(w.w1[e] >> 32) == want;
-      if (__ballot(!have) == 0) break;
-      if (polls >= ch.spin_limit) {
-        if (lane == 0) {
-          sh_fail[slot] = token;
-          __hip_atomic_fetch_add(&ch.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return __ballot(!have) == 0;
+    };
+    // (the first look stands in front of the loop, where the wait covers exactly the loads older than the words;
+    // at the head of a loop that asks again the compiler has to wait for every load of the wave)
+    if (!all_there()) {
+      for (int polls = 0;; ++polls) {
+        if (polls >= ch.spin_limit) {
+          if (lane == 0) {
+            sh_fail[slot] = token;
+            __hip_atomic_fetch_add(&ch.ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          return;
         }
-        return;
+        __builtin_amdgcn_s_sleep(1);
+        ask(k, w);
+        if (all_there()) break;
       }
-      __builtin_amdgcn_s_sleep(1);
-      ask(k, w);
     }
     if (G == 1 || grp == 0) {
 #pragma unroll

@@ -236,6 +236,7 @@ __global__ __launch_bounds__(256) void column_kernel(ColumnArgs p) {
 // segments into the value entering each segment, written where the map's b was.  The segments are
 // taken 1024 at a time: lane i takes the 16 segments [16 i, 16 i + 16) of the chunk, the wave scans
 // the 64 lane totals, and what leaves the chunk enters the next one.
+template <int UNUSED = 0>  // (a template so that every translation unit that includes this file may hold a copy)
 __global__ __launch_bounds__(256) void segment_carry_kernel(float* maps, long long numseq, int segments) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);

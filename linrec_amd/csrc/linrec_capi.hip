@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../include/linrec_hip.h"
+#include "kernel_table.hpp"
 #include "colblock_kernel.hpp"
 #include "coldrift_kernel.hpp"
 #include "column_kernel.hpp"
@@ -37,207 +38,22 @@ namespace {
 using linrec::ColumnArgs;
 using linrec::TileArgs;
 
-struct KernelEntry {
-  const char* name;
-  const void* fn;
-  int dtype, family, waves, slots, vec, mode, desc, carry;
-};
-
 // ---- kernel table ---------------------------------------------------------------------------
 // The reference compiles 116 configurations of 4 kernels and matches a runtime tuple against them
-// (linrec/impl/cuda/linrec.h:8-13, dispatch.h:53-72).  Here the table is a plain array of
-// instantiations; the planner below picks one entry from the problem shape.  TT is the storage type,
-// DT its LINREC_DTYPE_* code, PFX the prefix of the kernel's name; VEC is the number of elements of
-// a slot (16 bytes of TT, or 1).
-#define TILE_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC, CARRY)                                 \
-  {PFX "tile_w" #NW "_s" #S "_v" #VEC "_" #MODE "_" #DESC "_" #CARRY,                          \
-   (const void*)&linrec::tile_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, CARRY != 0>, DT, \
-   LINREC_FAMILY_TILE, NW, S, VEC, linrec::MODE, DESC, CARRY}
-#define TILE_ALL_DIRS(TT, DT, PFX, NW, S, VEC, CARRY)                                          \
-  TILE_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0, CARRY), TILE_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1, CARRY), \
-  TILE_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0, CARRY), TILE_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1, CARRY)
-#define CHAIN_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                       \
-  {PFX "chain_w" #NW "_s" #S "_v" #VEC "_" #MODE "_" #DESC,                                    \
-   (const void*)&linrec::chain_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_TILE, \
-   NW, S, VEC, linrec::MODE, DESC, 2}
-#define CHAIN_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
-  CHAIN_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), CHAIN_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
-  CHAIN_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), CHAIN_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
-#define TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
-  {PFX "team_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::team_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_TEAM, \
-   NW, S, VEC, linrec::MODE, DESC, 1}
-#define TEAM_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                                 \
-  TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
-  TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
-#define SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                       \
-  {PFX "sweep_w" #NW "_s" #S "_" #MODE "_" #DESC,                                              \
-   (const void*)&linrec::sweep_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_SWEEP, \
-   NW, S, VEC, linrec::MODE, DESC, 1}
-#define SWEEP_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
-  SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
-  SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), SWEEP_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
-// Tiles of loads in flight ahead of the scan: two in the backward with 16 waves of one slot, whose step loads
-// only 48 KB (one after the other in one process, us, against 8 waves of two slots with one tile ahead, which one
-// tile ahead in 16 waves had beaten by 1 to 4 %: 512 x 65536 112.4 against 117.5, 300 x 65536 68.3 against 71.2,
-// 16 x 1048576 60.1 against 63.6, 1 x 33554432 111.6 against 124.5); the forward gains nothing from it.
-#define DRIFT_TILES_AHEAD(NW, S, MODE) ((NW) == 16 && (S) == 1 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
-#define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
-  {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
-   NW, S, VEC, linrec::MODE, DESC, 1}
-#define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
-  DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
-#define DRIFT_BWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
-  DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
-#define TEAM_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                 \
-  TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), TEAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
-#define STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                      \
-  {PFX "stream_w" #NW "_s" #S "_" #MODE "_" #DESC,                                             \
-   (const void*)&linrec::stream_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_STREAM, \
-   NW, S, VEC, linrec::MODE, DESC, 0}
-#define STREAM_ALL_DIRS(TT, DT, PFX, NW, S, VEC)                                               \
-  STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1), \
-  STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), STREAM_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
-#define GROUP_ENTRY(TT, DT, PFX, VEC, MODE, DESC)                                              \
-  {PFX "group_v" #VEC "_" #MODE "_" #DESC,                                                     \
-   (const void*)&linrec::group_kernel<TT, VEC, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_GROUP, 4, 1, VEC, \
-   linrec::MODE, DESC, 0}
-#define GROUP_ALL_DIRS(TT, DT, PFX, VEC)                                                       \
-  GROUP_ENTRY(TT, DT, PFX, VEC, MODE_FWD, 0), GROUP_ENTRY(TT, DT, PFX, VEC, MODE_FWD, 1),      \
-  GROUP_ENTRY(TT, DT, PFX, VEC, MODE_BWD, 0), GROUP_ENTRY(TT, DT, PFX, VEC, MODE_BWD, 1)
-#define FLAT_ENTRY(TT, DT, PFX, VEC, S, MODE, DESC)                                            \
-  {PFX "flat_s" #S "_" #MODE "_" #DESC,                                                        \
-   (const void*)&linrec::flat_kernel<TT, VEC, S, linrec::MODE, DESC != 0>, DT, LINREC_FAMILY_FLAT, 4, S, VEC, \
-   linrec::MODE, DESC, 0}
-#define FLAT_ALL_DIRS(TT, DT, PFX, VEC, S)                                                     \
-  FLAT_ENTRY(TT, DT, PFX, VEC, S, MODE_FWD, 0), FLAT_ENTRY(TT, DT, PFX, VEC, S, MODE_FWD, 1),  \
-  FLAT_ENTRY(TT, DT, PFX, VEC, S, MODE_BWD, 0), FLAT_ENTRY(TT, DT, PFX, VEC, S, MODE_BWD, 1)
-#define COLUMN_ENTRY(TT, DT, PFX, VEC, U, MODE, DESC)                                          \
-  {PFX "column_v" #VEC "_u" #U "_" #MODE "_" #DESC,                                            \
-   (const void*)&linrec::column_kernel<TT, VEC, U, linrec::MODE, DESC != 0>, DT,               \
-   (VEC > 1 ? LINREC_FAMILY_COLUMN : LINREC_FAMILY_NAIVE), 4, U, VEC, linrec::MODE, DESC, 0}
-#define COLUMN_ALL_DIRS(TT, DT, PFX, VEC, U)                                                   \
-  COLUMN_ENTRY(TT, DT, PFX, VEC, U, MODE_FWD, 0), COLUMN_ENTRY(TT, DT, PFX, VEC, U, MODE_FWD, 1), \
-  COLUMN_ENTRY(TT, DT, PFX, VEC, U, MODE_BWD, 0), COLUMN_ENTRY(TT, DT, PFX, VEC, U, MODE_BWD, 1)
-
-// Column block kernels: the 16 waves of a workgroup share rows (the table's `carry` column holds the
-// number of lane groups a wave is split into: 1, 2 or 4).
-#define COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE, DESC)                                     \
-  {PFX "colblock_v" #VEC "_u" #U "_g" #G "_" #MODE "_" #DESC,                                  \
-   (const void*)&linrec::colblock_kernel<TT, VEC, U, 16, G, linrec::MODE, DESC != 0>, DT,      \
-   LINREC_FAMILY_COLUMN, 16, U, VEC, linrec::MODE, DESC, G}
-// Column drift kernels: column blocks in teams along the scan axis (`carry` column: lane groups per wave).
-#define COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE, DESC)                                    \
-  {PFX "coldrift_w" #NW "_v" #VEC "_u" #U "_" #MODE "_" #DESC,                                 \
-   (const void*)&linrec::coldrift_kernel<TT, VEC, U, NW, 1, linrec::MODE, DESC != 0>, DT,      \
-   LINREC_FAMILY_COLDRIFT, NW, U, VEC, linrec::MODE, DESC, 1}
-#define COLDRIFT_FWD_DIRS(TT, DT, PFX, NW, VEC, U)                                             \
-  COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_FWD, 0), COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_FWD, 1)
-#define COLDRIFT_BWD_DIRS(TT, DT, PFX, NW, VEC, U)                                             \
-  COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_BWD, 0), COLDRIFT_ENTRY(TT, DT, PFX, NW, VEC, U, MODE_BWD, 1)
-#define COLBLOCK_FWD_DIRS(TT, DT, PFX, VEC, U, G)                                              \
-  COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_FWD, 0), COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_FWD, 1)
-#define COLBLOCK_BWD_DIRS(TT, DT, PFX, VEC, U, G)                                              \
-  COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_BWD, 0), COLBLOCK_ENTRY(TT, DT, PFX, VEC, U, G, MODE_BWD, 1)
-
-// Segmented column launches: the reduce and the apply phase of one geometry (the table's `carry`
-// column holds the phase).
-#define SEGMENT_ENTRY(TT, DT, PFX, VEC, U, MODE, DESC, PH, PHNAME)                             \
-  {PFX "segment_" PHNAME "_v" #VEC "_u" #U "_" #MODE "_" #DESC,                                \
-   (const void*)&linrec::column_kernel<TT, VEC, U, linrec::MODE, DESC != 0, linrec::PH>, DT,   \
-   LINREC_FAMILY_SEGMENT, 4, U, VEC, linrec::MODE, DESC, linrec::PH}
-#define SEGMENT_PHASES(TT, DT, PFX, VEC, U, MODE, DESC)                                        \
-  SEGMENT_ENTRY(TT, DT, PFX, VEC, U, MODE, DESC, PHASE_REDUCE, "reduce"),                      \
-  SEGMENT_ENTRY(TT, DT, PFX, VEC, U, MODE, DESC, PHASE_APPLY, "apply")
-#define SEGMENT_ALL_DIRS(TT, DT, PFX, VEC, U)                                                  \
-  SEGMENT_PHASES(TT, DT, PFX, VEC, U, MODE_FWD, 0), SEGMENT_PHASES(TT, DT, PFX, VEC, U, MODE_FWD, 1), \
-  SEGMENT_PHASES(TT, DT, PFX, VEC, U, MODE_BWD, 0), SEGMENT_PHASES(TT, DT, PFX, VEC, U, MODE_BWD, 1)
-
-#define F32 float, LINREC_DTYPE_F32, ""
-#define F16 _Float16, LINREC_DTYPE_F16, "f16_"
-#define BF16 __bf16, LINREC_DTYPE_BF16, "bf16_"
-// indirection so that F32 / F16 / BF16 expand into three macro arguments
-#define TILE_(...) TILE_ALL_DIRS(__VA_ARGS__)
-#define CHAIN_(...) CHAIN_ALL_DIRS(__VA_ARGS__)
-#define TEAM_(...) TEAM_ALL_DIRS(__VA_ARGS__)
-#define SWEEP_(...) SWEEP_ALL_DIRS(__VA_ARGS__)
-#define DRIFT_FWD_(...) DRIFT_FWD_DIRS(__VA_ARGS__)
-#define DRIFT_BWD_(...) DRIFT_BWD_DIRS(__VA_ARGS__)
-#define TEAM_FWD_(...) TEAM_FWD_DIRS(__VA_ARGS__)
-#define STREAM_(...) STREAM_ALL_DIRS(__VA_ARGS__)
-#define COLUMN_(...) COLUMN_ALL_DIRS(__VA_ARGS__)
-#define GROUP_(...) GROUP_ALL_DIRS(__VA_ARGS__)
-#define FLAT_(...) FLAT_ALL_DIRS(__VA_ARGS__)
-#define SEGMENT_(...) SEGMENT_ALL_DIRS(__VA_ARGS__)
-#define COLDRIFT_FWD_(...) COLDRIFT_FWD_DIRS(__VA_ARGS__)
-#define COLDRIFT_BWD_(...) COLDRIFT_BWD_DIRS(__VA_ARGS__)
-#define COLBLOCK_FWD_(...) COLBLOCK_FWD_DIRS(__VA_ARGS__)
-#define COLBLOCK_BWD_(...) COLBLOCK_BWD_DIRS(__VA_ARGS__)
-
-// The 16-bit storage types get the geometries the planner picks for them (their register tiles are
-// twice as wide as fp32's, so two slots of eight elements per lane is the rule; the forward team
-// kernel, which keeps its prefetched tile packed, also comes with four).
-#define HALF_KERNELS(TY)                                                                        \
-  TILE_(TY, 1, 1, 8, 0), TILE_(TY, 2, 1, 8, 0), TILE_(TY, 4, 1, 8, 0), TILE_(TY, 4, 2, 8, 0),   \
-  TILE_(TY, 8, 2, 8, 0), TILE_(TY, 16, 2, 8, 0), TILE_(TY, 4, 2, 8, 1), TILE_(TY, 8, 4, 8, 1),  \
-  TILE_(TY, 4, 4, 1, 0), TILE_(TY, 4, 4, 1, 1), STREAM_(TY, 8, 2, 8), TEAM_(TY, 8, 2, 8),       \
-  TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8),                         \
-  GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
-  COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16),     \
-  SEGMENT_(TY, 4, 8), SEGMENT_(TY, 2, 8), SEGMENT_(TY, 1, 8),                             \
-  COLBLOCK_FWD_(TY, 2, 8, 1), COLBLOCK_BWD_(TY, 2, 4, 1), COLBLOCK_FWD_(TY, 2, 8, 2), COLBLOCK_BWD_(TY, 2, 4, 2)
-
-const KernelEntry kKernels[] = {
-    // one wave per row, rows up to 2048 elements
-    TILE_(F32, 1, 1, 4, 0), TILE_(F32, 1, 2, 4, 0), TILE_(F32, 1, 4, 4, 0), TILE_(F32, 1, 8, 4, 0),
-    // one workgroup per row
-    TILE_(F32, 2, 1, 4, 0), TILE_(F32, 2, 2, 4, 0), TILE_(F32, 2, 4, 4, 0), TILE_(F32, 4, 1, 4, 0),
-    TILE_(F32, 4, 2, 4, 0), TILE_(F32, 16, 2, 4, 0), TILE_(F32, 4, 4, 4, 0), TILE_(F32, 4, 8, 4, 0),
-    TILE_(F32, 8, 2, 4, 0), TILE_(F32, 8, 4, 4, 0), TILE_(F32, 16, 4, 4, 0),
-    // rows chained over several workgroups by look-back
-    TILE_(F32, 1, 4, 4, 1), TILE_(F32, 4, 2, 4, 1), TILE_(F32, 4, 4, 4, 1), TILE_(F32, 4, 8, 4, 1),
-    TILE_(F32, 8, 4, 4, 1), TILE_(F32, 8, 8, 4, 1), TILE_(F32, 16, 4, 4, 1),
-    // tensors whose base addresses disagree modulo 16 bytes: element-sized accesses
-    TILE_(F32, 4, 4, 1, 0), TILE_(F32, 4, 4, 1, 1),
-    // look-back with several tiles (of different rows) per workgroup, next tile prefetched
-    CHAIN_(F32, 4, 2, 4), CHAIN_(F32, 4, 4, 4), CHAIN_(F32, 8, 2, 4), CHAIN_(F32, 8, 4, 4),
-    // one workgroup walks a whole row
-    STREAM_(F32, 4, 4, 4), STREAM_(F32, 8, 2, 4), STREAM_(F32, 8, 4, 4), STREAM_(F32, 16, 2, 4), STREAM_(F32, 8, 8, 4),
-    // several workgroups walk one row side by side
-    TEAM_(F32, 4, 2, 4), TEAM_(F32, 4, 4, 4), TEAM_(F32, 8, 2, 4), TEAM_(F32, 8, 4, 4),
-    // teams that go on from row to row so that the launch reads the tensors front to back
-    SWEEP_(F32, 8, 4, 4), SWEEP_(F32, 8, 2, 4), SWEEP_(F32, 4, 4, 4), SWEEP_(F32, 8, 8, 4),
-    // the same launch shape with a tile stored two steps late, so that nobody waits for the exchange
-    DRIFT_FWD_(F32, 8, 4, 4), DRIFT_FWD_(F32, 8, 2, 4), DRIFT_BWD_(F32, 8, 2, 4), DRIFT_FWD_(F32, 4, 4, 4),
-    // (16 waves of two slots forward: the 128 registers to be had suffice for teams of at most 64)
-    DRIFT_BWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 1, 4), DRIFT_FWD_(F32, 16, 2, 4),
-    // short rows: several rows per wave
-    GROUP_(F32, 4),
-    // short rows that are not whole slots, dense: the tensor as one flat array
-    FLAT_(F32, 4, 4), FLAT_(F32, 4, 2),
-    // strided scan axis
-    COLUMN_(F32, 4, 4), COLUMN_(F32, 4, 8),
-    COLUMN_(F32, 2, 8), COLUMN_(F32, 2, 16), COLUMN_(F32, 1, 4), COLUMN_(F32, 1, 8), COLUMN_(F32, 1, 16),
-    // strided scan axis, few rows: the scan axis cut into segments (reduce, carry, apply)
-    SEGMENT_(F32, 4, 8), SEGMENT_(F32, 2, 8), SEGMENT_(F32, 1, 8), SEGMENT_(F32, 1, 16),
-    // strided scan axis, a few thousand to a few ten thousand rows: the waves of a workgroup share rows
-    // (two rows per lane: the backward holds three tensors, so it takes runs of 4 positions to stay in registers)
-    COLBLOCK_FWD_(F32, 1, 8, 1), COLBLOCK_BWD_(F32, 1, 8, 1), COLBLOCK_FWD_(F32, 2, 8, 1), COLBLOCK_BWD_(F32, 2, 4, 1),
-    // fewer rows: waves split into 2 groups of lanes that share rows (128-byte accesses; 4 groups of 16
-    // floats run at half the rate: 4096 x 8192 151.8 / 270.7 us against 101.1 / 168.7 us)
-    COLBLOCK_FWD_(F32, 1, 8, 2), COLBLOCK_BWD_(F32, 1, 8, 2), COLBLOCK_FWD_(F32, 2, 8, 2), COLBLOCK_BWD_(F32, 2, 4, 2),
-    // strided scan axis, a few hundred to a few thousand rows: column blocks in teams along the scan axis
-    // (the backward holds three tensors of four steps: runs of 4 positions)
-    // (two rows per lane and runs of 8 positions in 8 waves were compiled and lost: 4096 x 16384 189 / 276 us)
-    // (nor two rows per lane with runs of 4 positions in 16 waves, whose 512-byte accesses a memory-only kernel
-    // likes better by 14 %: twice the team and half the positions per step make four times the exchange,
-    // 4096 x 16384 forward 187 against 157 us, 2048 x 16384 124 against 85.3 us, 8192 x 4096 89.6 against 82.7 us)
-    COLDRIFT_FWD_(F32, 16, 1, 8), COLDRIFT_BWD_(F32, 16, 1, 4), COLDRIFT_FWD_(F32, 8, 1, 16), COLDRIFT_BWD_(F32, 8, 1, 16),
-    // fp16 and bf16 storage (fp32 arithmetic)
-    HALF_KERNELS(F16), HALF_KERNELS(BF16),
-};
-constexpr int kNumKernels = int(sizeof(kKernels) / sizeof(kKernels[0]));
+// (linrec/impl/cuda/linrec.h:8-13, dispatch.h:53-72).  Here the table is a plain array of instantiations
+// (kernel_table.hpp), compiled in groups (kernels_*.hip) and put together once when the library is loaded;
+// the planner below picks one entry from the problem shape.
+using linrec::KernelEntry;
+const std::vector<KernelEntry> g_kernel_table = [] {
+  std::vector<KernelEntry> all;
+  for (const linrec::KernelGroup g : {linrec::kernels_f32_rows(), linrec::kernels_f32_walk(), linrec::kernels_f32_teams(), linrec::kernels_f32_cols(),
+                                      linrec::kernels_f16_rows(), linrec::kernels_f16_cols(), linrec::kernels_bf16_rows(),
+                                      linrec::kernels_bf16_cols()})
+    all.insert(all.end(), g.entries, g.entries + g.count);
+  return all;
+}();
+const KernelEntry* const kKernels = g_kernel_table.data();
+const int kNumKernels = int(g_kernel_table.size());
 
 int find_kernel(int dtype, int family, int waves, int slots, int vec, int mode, int desc, int carry) {
   for (int i = 0; i < kNumKernels; ++i) {
@@ -348,7 +164,24 @@ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Stream kernels take over from tiles for rows of more than 2048 slots once there are enough rows
 // to give every CU work.
 constexpr int64_t kLongRowSlots = 2048;  // 8192 floats, 16384 halves
-constexpr int64_t kStreamMinRows = 129;   // (these three on 256 CUs; scaled by Problem::at)
+
+// The crossovers between the long-row kernels come from a generated table (plan_thresholds.inc, written by the
+// tuning harness from timings on the device): kT_<name> below, and by name through linrec_plan_threshold.
+struct PlanThreshold {
+  const char* name;
+  int64_t value;
+};
+#define LINREC_THRESHOLD(name, value) constexpr int64_t kT_##name = value;
+#include "plan_thresholds.inc"
+#undef LINREC_THRESHOLD
+#define LINREC_THRESHOLD(name, value) {#name, value},
+constexpr PlanThreshold kPlanThresholds[] = {
+#include "plan_thresholds.inc"
+};
+#undef LINREC_THRESHOLD
+constexpr int kNumPlanThresholds = int(sizeof(kPlanThresholds) / sizeof(kPlanThresholds[0]));
+
+constexpr int64_t kStreamMinRows = kT_stream_min_rows;   // (these three on 256 CUs; scaled by Problem::at)
 constexpr int64_t kSplitBelowRows = 192;  // rows of a few thousand elements are cut into look-back tiles below this
 constexpr int64_t kSweepBelowRows = 192;  // sweep kernels take 16 .. 191 rows, stream kernels 192 .. 256
 // Fewer long rows: teams of workgroups per row, sized so that at most one workgroup per CU runs
@@ -421,7 +254,7 @@ int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int6
 // 128 x 65536 20.1 / 33.2 against 19.9 / 29.4, 120 x 65536 18.9 / 32.4 against 18.6 / 27.9, 150 x 49152
 // 18.1 / 33.3 against 18.4 / 25.7; 200 x 32768 18.2 / 28.5 against 15.2 / 22.3 for one workgroup per row.
 bool little_work_in_many_rows(const Problem& q) {
-  return q.dtype == LINREC_DTYPE_F32 && q.numseq * 4 >= q.cus && q.numseq * q.seqlen <= 4 * 8192 * q.cus;
+  return q.dtype == LINREC_DTYPE_F32 && q.numseq * 4 >= q.cus && q.numseq * q.seqlen <= kT_little_work_max_tiles_per_cu * 8192 * q.cus;
 }
 // The largest team a drift kernel of this geometry serves: a lane of a wave per team mate, in every wave - except
 // 16 waves of two slots, compiled for one collecting wave.
@@ -444,13 +277,15 @@ int drift_slots_for(const Problem& q, int fv) {
   // 4096 x 65536 532.2 / 948.0 against 543.9 / 934.5 (tiles of 8192 in 16 waves of two slots: 271.0, 569.5, 391.9,
   // 540.6 forward).
   const bool many_rows = q.numseq > q.at(2048);
-  if (many_rows && q.is_bwd) return 0;
+  if (q.is_bwd && q.numseq > q.at(kT_drift_bwd_max_rows)) return 0;
   // The backward of 16 to 127 rows with little work in all stays with the sweep kernels' tiles of 16384 elements
   // (24 x 262144 25.3 against 26.3 us, 40 x 196608 27.0 against 30.8 us; but 100 x 131072 55.1 against 48.5 us,
   // 16 x 1048576 63.5 against 61.9 us, 32 x 1048576 123.1 against 118.0 us, 64 x 524288 118.3 against 116.3 us -
   // all with one tile of loads ahead; with two, 64 x 524288 takes 112.6 us, 256 x 262144 219.7 against 232.8 us and
   // 512 x 262144 453.1 against 452.3 us).
-  if (q.is_bwd && q.numseq * 16 >= q.cus && q.numseq < q.at(128) && q.numseq * q.seqlen < 6 * 8192 * q.cus) return 0;
+  if (q.is_bwd && q.numseq * 16 >= q.cus && q.numseq < q.at(128) &&
+      q.numseq * q.seqlen < kT_drift_bwd_few_rows_min_tiles_per_cu * 8192 * q.cus)
+    return 0;
   if (little_work_in_many_rows(q)) return 0;
   for (int s : {4, 2, 1}) {
     if (half != (s == 1)) continue;
@@ -469,7 +304,8 @@ int drift_slots_for(const Problem& q, int fv) {
     // 2048 x 16384 68.9 / 120.0 against 70.4 / 117.4)
     // (with 16 waves and two tiles of loads ahead the backward of 512 rows and more gains from four such tiles on:
     // 2048 x 16384 111.8 against 119.0 us, 768 x 16384 43.9 against 45.5 us)
-    if (s == 2 && tiles_per_row < 8 && !(q.is_bwd && q.numseq >= q.at(512))) continue;
+    if (s == 2 && tiles_per_row < kT_drift_min_small_tiles_per_row && !(q.is_bwd && q.numseq >= q.at(kT_drift_bwd_short_rows_min_rows)))
+      continue;
     // the teams have to fill at least half the chip, and every member gets a few tiles (1 x 4194304 in four
     // steps of 4096 elements: 16.4 / 19.8 us, what look-back tiles take)
     if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < (s == 4 ? 3 : 4) * q.cus) continue;
@@ -528,7 +364,7 @@ int sweep_slots_for(const Problem& q, int fv) {
 }
 constexpr int64_t kTailMaxRows = 96;  // rows beyond one per CU that a second launch takes (on 256 CUs)
 constexpr int64_t kGroupMaxSlots = 32;  // rows up to this many slots are packed several to a wave
-constexpr int64_t kTeamMinRows = 6;
+constexpr int64_t kTeamMinRows = kT_team_min_rows;
 // 16-bit storage, forward: teams of 64 already win from three rows on (bf16 3 x 4194304 28.0 against 40.3 us for
 // look-back tiles, 4 x 8388608 55.1 against 85.6 us, 5 x 2097152 21.7 against 35.0 us; the backward is a tie:
 // 3 x 4194304 48.7 against 46.4 us, 4 x 8388608 103.7 against 100.1 us)
@@ -1358,7 +1194,7 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
     const dim3 grid((unsigned)plan.grid), block((unsigned)plan.block);
     hipError_t e = hipLaunchKernel(kKernels[reduce_id].fn, grid, block, args, 0, stream);
     if (e != hipSuccess) return int(e);
-    linrec::segment_carry_kernel<<<dim3((unsigned)ceil_div(q.numseq, 4)), dim3(256), 0, stream>>>(a.maps, q.numseq, int(segments));
+    linrec::segment_carry_kernel<><<<dim3((unsigned)ceil_div(q.numseq, 4)), dim3(256), 0, stream>>>(a.maps, q.numseq, int(segments));
     e = hipLaunchKernel(k.fn, grid, block, args, 0, stream);
     return e == hipSuccess ? int(hipGetLastError()) : int(e);
   }
@@ -1725,6 +1561,16 @@ int linrec_set_spin_limit(int polls) {
 // wall clock at their phase boundaries (NULL switches stamping off).
 void linrec_debug_set_timing_buffer(unsigned long long* device_buffer) { g_timing_buffer = device_buffer; }
 #endif
+
+int linrec_plan_threshold_count(void) { return kNumPlanThresholds; }
+
+const char* linrec_plan_threshold_name(int index) {
+  return index >= 0 && index < kNumPlanThresholds ? kPlanThresholds[index].name : nullptr;
+}
+
+int64_t linrec_plan_threshold_value(int index) {
+  return index >= 0 && index < kNumPlanThresholds ? kPlanThresholds[index].value : -1;
+}
 
 int linrec_kernel_count(void) { return kNumKernels; }
 

@@ -3,7 +3,9 @@
 Counterpart of the reference's eval/tune.py:58-134 (grid search over compiled configurations with
 time, throughput and difference to a reference) and eval/func_attrs.py:25-60 (register / spill
 report).  Every compiled geometry that can serve the shape is timed with HIP events on rotating
-buffer sets and checked against the library's default choice for that shape.
+buffer sets and checked against the library's sequential host loop in float64 on the same values
+(max|difference| / max|reference|), as the reference checks every configuration against its
+one-thread-per-row kernel (eval/tune.py:98-102).
 
     python -m linrec_amd.tune --shape 512 65536 [--dtype f32|f16|bf16] [--reverse] [--transposed] [--mixed-phase]
                               [--only TEXT] [--attrs] [--csv out.csv]
@@ -101,6 +103,21 @@ def _event_ms(fn, iters, warmup):
 DTYPES = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 
 
+def sequential_reference(x, c, dy, reverse):
+    """outputs, d_inputs, d_coeffs of the library's sequential host loop (linrec_host_fwd_f64 / _bwd_f64) in
+    float64 on the values of the device tensors x, c, dy: float64 CPU tensors."""
+    xh, ch, dyh = (t.detach().to("cpu", torch.float64) for t in (x, c, dy))
+    y = nat.fwd(xh, ch, reverse)
+    dx, dc = nat.bwd(dyh, ch, y, reverse)
+    return y, dx, dc
+
+
+def normwise_error(got, want64):
+    """max|got - want| / max|want| in float64 (the figure the parity tests are written in)."""
+    scale = want64.abs().max().item()
+    return (got.double() - want64).abs().max().item() / (scale if scale > 0 else 1.0)
+
+
 def sweep(shape, reverse=False, transposed=False, sets=3, iters=50, warmup=10, device="cuda:0", dtype=torch.float32,
           mixed_phase=False, only=None):
     """List of dict rows: one per candidate geometry, forward and backward time and GB/s (a pass a
@@ -121,10 +138,13 @@ def sweep(shape, reverse=False, transposed=False, sets=3, iters=50, warmup=10, d
             c = buf[1:1 + n].view(shape).copy_(c)
         y, dx, dc = (torch.empty_strided(x.size(), x.stride(), dtype=dtype, device=dev) for _ in range(3))
         bufs.append((x, c, dy, y, dx, dc))
-    ref_y = nat.fwd(bufs[0][0], bufs[0][1], reverse)
-    ref_dx, ref_dc = nat.bwd(bufs[0][2], bufs[0][1], ref_y, reverse)
+    # Every candidate is checked against the library's sequential host loop in float64 on the same values (the
+    # role of the one-thread-per-row kernel in the reference's grid search, eval/tune.py:98-102): a float64
+    # recurrence that shares no code with the device kernels.
+    ref_y, ref_dx, ref_dc = (t.to(dev) for t in sequential_reference(bufs[0][0], bufs[0][1], bufs[0][2], reverse))
+    saved_y = ref_y.to(dtype)  # the saved outputs the backward passes run on
     for b in bufs:
-        b[3].copy_(nat.fwd(b[0], b[1], reverse))  # the saved outputs the backward passes are timed on
+        b[3].copy_(nat.fwd(b[0], b[1], reverse))
     names = nat.kernel_table()
     rows = []
     for label, tun in candidates(bufs[0][0]):
@@ -136,25 +156,25 @@ def sweep(shape, reverse=False, transposed=False, sets=3, iters=50, warmup=10, d
             if tun is not None and pl["family"] != tun.family:
                 raise NotImplementedError
             y = nat.fwd(bufs[0][0], bufs[0][1], reverse, tun)
-            diff = (y.float() - ref_y.float()).abs().max().item()
+            diff = normwise_error(y, ref_y)
             f = _event_ms(lambda i: nat.fwd(bufs[i % sets][0], bufs[i % sets][1], reverse, tun, out=bufs[i % sets][4]),
                           iters, warmup)
             row.update(kernel=names[pl["kernel_id"]], grid=pl["grid"], team=pl["tasks"], fwd_us=f * 1e3,
-                       fwd_GBps=3 * es * n / f / 1e6, fwd_maxabs_vs_default=diff)
+                       fwd_GBps=3 * es * n / f / 1e6, fwd_err_vs_sequential=diff)
         except (RuntimeError, NotImplementedError):
-            row.update(kernel="-", grid=0, team=0, fwd_us=float("nan"), fwd_GBps=float("nan"), fwd_maxabs_vs_default=float("nan"))
+            row.update(kernel="-", grid=0, team=0, fwd_us=float("nan"), fwd_GBps=float("nan"), fwd_err_vs_sequential=float("nan"))
         try:
             pl = nat.plan(bufs[0][0], reverse, True, tun)
             if tun is not None and pl["family"] != tun.family:
                 raise NotImplementedError
-            dx, dc = nat.bwd(bufs[0][2], bufs[0][1], ref_y, reverse, tun)
-            diff = max((a.float() - b.float()).abs().max().item() for a, b in ((dx, ref_dx), (dc, ref_dc)))
+            dx, dc = nat.bwd(bufs[0][2], bufs[0][1], saved_y, reverse, tun)
+            diff = max(normwise_error(dx, ref_dx), normwise_error(dc, ref_dc))
             b = _event_ms(lambda i: nat.bwd(bufs[i % sets][2], bufs[i % sets][1], bufs[i % sets][3], reverse, tun,
                                             out=(bufs[i % sets][4], bufs[i % sets][5])), iters, warmup)
             row.update(bwd_kernel=names[pl["kernel_id"]], bwd_team=pl["tasks"], bwd_us=b * 1e3, bwd_GBps=5 * es * n / b / 1e6,
-                       bwd_maxabs_vs_default=diff)
+                       bwd_err_vs_sequential=diff)
         except (RuntimeError, NotImplementedError):
-            row.update(bwd_kernel="-", bwd_team=0, bwd_us=float("nan"), bwd_GBps=float("nan"), bwd_maxabs_vs_default=float("nan"))
+            row.update(bwd_kernel="-", bwd_team=0, bwd_us=float("nan"), bwd_GBps=float("nan"), bwd_err_vs_sequential=float("nan"))
         if row["kernel"] != "-" or row["bwd_kernel"] != "-":
             rows.append(row)
     return rows
