@@ -369,6 +369,7 @@ constexpr int64_t kTeamMinRows = kT_team_min_rows;
 // look-back tiles, 4 x 8388608 55.1 against 85.6 us, 5 x 2097152 21.7 against 35.0 us; the backward is a tie:
 // 3 x 4194304 48.7 against 46.4 us, 4 x 8388608 103.7 against 100.1 us)
 constexpr int64_t kTeamMinRowsHalfFwd = 3;
+constexpr int64_t kTeamMinRowsHalfBwd = 6;
 
 // Rows one lane of a column kernel takes: 8 bytes' worth (measured best on 262144 x 256: fp32 two
 // rows 131 / 220 us against 132 / 236 us for four; bf16 four rows 70 / 114 us against 101 / 146 us
@@ -605,7 +606,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
         if (drift_slots_for(q, fv) > 0) family = LINREC_FAMILY_DRIFT;
         else if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
         else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) family = LINREC_FAMILY_STREAM;
-        else if (q.numseq >= (half && !q.is_bwd ? kTeamMinRowsHalfFwd : kTeamMinRows)) family = LINREC_FAMILY_TEAM;
+        else if (q.numseq >= (half ? (q.is_bwd ? kTeamMinRowsHalfBwd : kTeamMinRowsHalfFwd) : kTeamMinRows)) family = LINREC_FAMILY_TEAM;
       }
       // 16-bit storage, many rows of exactly two of the stream kernel's tiles (16384 elements): one workgroup of
       // 8 waves that walks the row beats one tile of 16 waves (bf16 2048 x 16384 34.1 / 57.0 against 36.4 / 59.7 us,

@@ -10,8 +10,13 @@ one-thread-per-row kernel (eval/tune.py:98-102).
     python -m linrec_amd.tune --shape 512 65536 [--dtype f32|f16|bf16] [--reverse] [--transposed] [--mixed-phase]
                               [--only TEXT] [--attrs] [--csv out.csv]
     python -m linrec_amd.tune --memory-probe [--shape 512 65536]
+    python -m linrec_amd.tune --write-table [PATH]
 
 `--only TEXT` keeps the geometries whose label contains TEXT (one kernel under a profiler).
+`--write-table` measures the crossovers between the long-row kernels that the launch planner decides by (one
+sweep per threshold: the two kernels on either side, timed over a range of the quantity the rule is written in)
+and writes them as csrc/plan_thresholds.inc, the file the planner is compiled with - the counterpart of the
+dispatch table the reference's grid search writes (eval/tune.py:104-134).  Without PATH the file is printed.
 `--memory-probe` times no scan at all: the memory-only kernel with a pass's mix of streams (2 in and 1 out,
 3 in and 2 out) over tensors of the given size, its 16 KiB blocks launched in address order and in orders
 that keep some address bits the same among the blocks in flight, which is what a launch with one
@@ -206,6 +211,155 @@ def memory_probe(shape, sets=3, iters=40, warmup=8, device="cuda:0"):
     return rows
 
 
+
+# ---- the planner's crossover thresholds ------------------------------------------------------------
+class Crossover:
+    """One threshold of the planner: `name` in csrc/plan_thresholds.inc, the swept `values` of the quantity the
+    rule is written in, `shape(v)` -> (rows, length) of the problem timed at v, the tunings on either side
+    ({pass: Tuning}; `low` serves the small values - the fastest of a list, where the planner has several kernels to
+    fall back on - and `high` the large ones) and the passes whose times are added.
+    kind 'first_high': the threshold is the smallest value from which `high` is faster on all larger values
+    tried; 'last_low': the largest value up to which `low` is at least as fast on all smaller values tried."""
+
+    def __init__(self, name, what, values, shape, low, high, passes=("fwd", "bwd"), kind="first_high"):
+        self.name, self.what, self.values, self.shape = name, what, values, shape
+        self.low, self.high, self.passes, self.kind = low, high, passes, kind
+
+
+def _t(family, waves=0, slots=0, carry=-1, tasks=0):
+    return nat.Tuning(family, waves, slots, carry, tasks)
+
+
+def _both(t):
+    return {"fwd": t, "bwd": t}
+
+
+_DRIFT = {"fwd": _t(nat.FAMILY_DRIFT, 16, 2), "bwd": _t(nat.FAMILY_DRIFT, 16, 1)}
+_DRIFT_SMALL = {"fwd": _t(nat.FAMILY_DRIFT, 16, 1), "bwd": _t(nat.FAMILY_DRIFT, 16, 1)}
+
+CROSSOVERS = [
+    Crossover("stream_min_rows", "ragged long rows (65540 elements): one team of workgroups per row against one "
+              "workgroup per row, by the number of rows", [64, 96, 112, 128, 129, 144, 160, 192],
+              lambda v: (v, 65540), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_STREAM))),
+    Crossover("team_min_rows", "a few ragged very long rows (1048580 elements): look-back tiles against one team of "
+              "64 workgroups per row, by the number of rows", [2, 3, 4, 5, 6, 8, 12],
+              lambda v: (v, 1048580), _both(_t(nat.FAMILY_TILE, 8, 8, 1, 1)), _both(_t(nat.FAMILY_TEAM))),
+    Crossover("drift_bwd_max_rows", "backward of many rows of 32768 elements: drift teams (tiles stored two steps "
+              "late) against sweep teams (tiles of 8192 elements, exchange waited for), by the number of rows",
+              [1024, 1536, 2048, 3072, 4096], lambda v: (v, 32768), _DRIFT_SMALL, _both(_t(nat.FAMILY_SWEEP, 8, 4)),
+              passes=("bwd",), kind="last_low"),
+    Crossover("drift_bwd_few_rows_min_tiles_per_cu", "backward of 32 long rows: sweep teams with tiles of 16384 "
+              "elements against drift teams, by the tiles of 8192 elements per compute unit",
+              [2, 3, 4, 6, 8, 12, 16], lambda v: (32, v * 65536), _both(_t(nat.FAMILY_SWEEP, 8, 8)), _DRIFT_SMALL,
+              passes=("bwd",)),
+    Crossover("little_work_max_tiles_per_cu", "128 rows with little work: sweep teams with tiles of 16384 elements "
+              "against drift teams, by the tiles of 8192 elements per compute unit", [2, 4, 6, 8, 12],
+              lambda v: (128, v * 16384), _both(_t(nat.FAMILY_SWEEP, 8, 8)), _DRIFT, kind="last_low"),
+    Crossover("drift_min_small_tiles_per_row", "forward of 600 rows that are whole tiles of 4096 elements but not of "
+              "8192: one workgroup per row, or sweep teams, against drift teams, by the tiles of a row", [5, 7, 9, 11, 13, 15, 17],
+              lambda v: (600, v * 4096), [_both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))], _DRIFT_SMALL,
+              passes=("fwd",)),
+    Crossover("drift_bwd_short_rows_min_rows", "backward of rows of four tiles of 4096 elements: one workgroup per "
+              "row against drift teams, by the number of rows", [128, 256, 384, 512, 768, 1024, 2048],
+              lambda v: (v, 16384), _both(_t(nat.FAMILY_STREAM)), _DRIFT_SMALL, passes=("bwd",)),
+]
+
+
+def _time_tunings(shape, tunings, passes, sets=3, iters=30, warmup=6, device="cuda:0", rounds=2):
+    """Microseconds of the listed passes added up, for each {pass: Tuning} of `tunings` on tensors of `shape`
+    (the candidates take turns, the least of `rounds` counts); inf where the library has no such kernel."""
+    dev = torch.device(device)
+    bufs = []
+    for _ in range(sets):
+        x, c, dy = (f(shape, device=dev) for f in (torch.randn, torch.rand, torch.randn))
+        y = nat.fwd(x, c)
+        bufs.append((x, c, dy, y, torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)))
+    best = [float("inf")] * len(tunings)
+    for _ in range(rounds):
+        for k, tun in enumerate(tunings):
+            total = 0.0
+            try:
+                for p in passes:
+                    pl = nat.plan(bufs[0][0], False, p == "bwd", tun[p])
+                    if pl["family"] != tun[p].family:
+                        raise NotImplementedError
+                    if p == "fwd":
+                        total += _event_ms(lambda i: nat.fwd(bufs[i % sets][0], bufs[i % sets][1], False, tun[p], out=bufs[i % sets][4]),
+                                           iters, warmup) * 1e3
+                    else:
+                        total += _event_ms(lambda i: nat.bwd(bufs[i % sets][2], bufs[i % sets][1], bufs[i % sets][3], False, tun[p],
+                                                             out=(bufs[i % sets][5], bufs[i % sets][6])), iters, warmup) * 1e3
+            except (RuntimeError, NotImplementedError):
+                total = float("inf")
+            best[k] = min(best[k], total)
+    return best
+
+
+def measure_crossover(x, log=None):
+    """(threshold, [(value, shape, us_low, us_high)]) of one Crossover on the current device."""
+    rows = []
+    for v in x.values:
+        lows = x.low if isinstance(x.low, list) else [x.low]
+        times = _time_tunings(x.shape(v), lows + [x.high], x.passes)
+        lo, hi = min(times[:-1]), times[-1]
+        rows.append((v, x.shape(v), lo, hi))
+        if log:
+            log(f"{x.name}: {v} {x.shape(v)} low {lo:.1f} us high {hi:.1f} us")
+    high_wins = [hi < lo for _, _, lo, hi in rows]
+    if x.kind == "first_high":
+        k = len(rows)
+        while k > 0 and high_wins[k - 1]:
+            k -= 1
+        # (never faster: one past the largest value tried)
+        threshold = rows[k][0] if k < len(rows) else rows[-1][0] + 1
+    else:
+        k = 0
+        while k < len(rows) and not high_wins[k]:
+            k += 1
+        # (never at least as fast: one below the smallest value tried)
+        threshold = rows[k - 1][0] if k > 0 else rows[0][0] - 1
+    return threshold, rows
+
+
+TABLE_HEADER = """// Crossover thresholds of the launch planner for long rows on the unit-stride axis (fp32), on the full part (256
+// compute units; the planner scales row counts to the device in hand).
+//
+// GENERATED by `python -m linrec_amd.tune --write-table` (the counterpart of the table the reference's grid search
+// writes, eval/tune.py:104-134): every line is the smallest value of the swept quantity from which the second
+// kernel was faster than the first on all larger values tried (or the largest up to which the first held its own);
+// the timings behind each line stand above it.  Edit by re-running the command on the device, not by hand.
+//
+// LINREC_THRESHOLD(name, value)
+"""
+
+
+def write_table(path=None, only=None, log=None):
+    """Measures every Crossover and returns the text of csrc/plan_thresholds.inc (written to `path` if given).
+    `only`: names to measure; the others keep the values the library is compiled with."""
+    current = nat.plan_thresholds()
+    device = torch.cuda.get_device_name(0)
+    out = [TABLE_HEADER.rstrip("\n"), f"// measured on: {device}, {nat.lib().linrec_compute_units()} compute units"]
+    for x in CROSSOVERS:
+        out.append("//")
+        out.append(f"// {x.name}: {x.what}")
+        if only is not None and x.name not in only:
+            out.append("// (not measured in this run: value kept)")
+            out.append(f"LINREC_THRESHOLD({x.name}, {current[x.name]})")
+            continue
+        threshold, rows = measure_crossover(x, log)
+        passes = " + ".join(x.passes)
+        for v, shape, lo, hi in rows:
+            out.append(f"//   {v:>6}  {shape[0]} x {shape[1]}: {passes} {lo:.1f} us against {hi:.1f} us")
+        out.append(f"LINREC_THRESHOLD({x.name}, {threshold})")
+    missing = set(current) - {x.name for x in CROSSOVERS}
+    assert not missing, f"thresholds without a sweep: {missing}"
+    text = "\n".join(out) + "\n"
+    if path:
+        with open(path, "w") as f:
+            f.write(text)
+    return text
+
+
 def attrs_report():
     """numRegs / LDS / scratch of every compiled kernel (hipFuncGetAttributes)."""
     return [dict(kernel=name, **nat.kernel_attrs(i)) for i, name in enumerate(nat.kernel_table())]
@@ -223,8 +377,17 @@ def main(argv=None):
     ap.add_argument("--memory-probe", action="store_true",
                     help="time the memory-only kernel with address bits held among the blocks in flight instead")
     ap.add_argument("--attrs", action="store_true", help="print the register / LDS / scratch table instead")
+    ap.add_argument("--write-table", nargs="?", const="-", default=None, metavar="PATH",
+                    help="measure the planner's crossover thresholds and write csrc/plan_thresholds.inc (to PATH, or print it)")
+    ap.add_argument("--thresholds", nargs="*", default=None, metavar="NAME", help="with --write-table: only these thresholds")
     ap.add_argument("--csv", default=None)
     a = ap.parse_args(argv)
+    if a.write_table is not None:
+        text = write_table(None if a.write_table == "-" else a.write_table, a.thresholds,
+                           log=lambda m: print(m, file=sys.stderr, flush=True))
+        if a.write_table == "-":
+            print(text, end="")
+        return
     if a.attrs:
         rows = attrs_report()
     elif a.memory_probe:

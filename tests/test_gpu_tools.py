@@ -74,6 +74,23 @@ def test_every_tuning_candidate_matches_the_oracle(shape, transposed):
     assert nat.gave_up_count() == 0
 
 
+def test_write_table_measures_a_crossover_and_keeps_the_rest(tmp_path):
+    """`python -m linrec_amd.tune --write-table`: the file the planner is compiled with, one threshold measured
+    again here, the others kept."""
+    import re
+    from linrec_amd import _native as nat, tune
+    path = tmp_path / "plan_thresholds.inc"
+    text = tune.write_table(str(path), only=["team_min_rows"])
+    assert path.read_text() == text and text.startswith(tune.TABLE_HEADER)
+    got = {m.group(1): int(m.group(2)) for m in re.finditer(r"^LINREC_THRESHOLD\((\w+), (-?\d+)\)", text, flags=re.M)}
+    cur = nat.plan_thresholds()
+    assert set(got) == set(cur)
+    assert all(got[k] == cur[k] for k in cur if k != "team_min_rows")
+    x = next(c for c in tune.CROSSOVERS if c.name == "team_min_rows")
+    assert x.values[0] - 1 <= got["team_min_rows"] <= x.values[-1] + 1
+    assert text.count(" us against ") == len(x.values) and text.count("value kept") == len(cur) - 1
+
+
 def test_memory_probe_reports_every_launch_order():
     from linrec_amd import tune
     rows = tune.memory_probe((64, 16384), sets=1, iters=3, warmup=1)

@@ -20,13 +20,28 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "linrec_hip.h")).read()
-    declared = set(re.findall(r"^\s*(?:int|size_t|const char\*|void)\s+(linrec_\w+)\s*\(", header, flags=re.M))
-    assert len(declared) == 29, declared
+    declared = set(re.findall(r"^\s*(?:int|int64_t|size_t|const char\*|void)\s+(linrec_\w+)\s*\(", header, flags=re.M))
+    assert len(declared) == 32, declared
     lib = ctypes.CDLL(nat.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/linrec_hip.h but not exported"
     assert declared == set(nat.EXPORTS), (declared ^ set(nat.EXPORTS))
     assert lib.linrec_hip_abi_version() == 1
+
+
+def test_planner_thresholds_come_from_the_generated_table():
+    """csrc/plan_thresholds.inc (written by `python -m linrec_amd.tune --write-table`) is what the library is compiled
+    with, every threshold in it has a sweep in the harness that can measure it again, and the file carries the
+    timings it was derived from."""
+    from linrec_amd import tune
+    text = open(os.path.join(ROOT, "linrec_amd", "csrc", "plan_thresholds.inc")).read()
+    in_file = {m.group(1): int(m.group(2)) for m in re.finditer(r"^LINREC_THRESHOLD\((\w+), (-?\d+)\)", text, flags=re.M)}
+    assert in_file == nat.plan_thresholds() and len(in_file) >= 7
+    assert {x.name for x in tune.CROSSOVERS} == set(in_file)
+    assert text.startswith(tune.TABLE_HEADER) and "measured on:" in text
+    for x in tune.CROSSOVERS:  # (the lines of timings above each value)
+        block = text[text.index(f"// {x.name}:"):text.index(f"LINREC_THRESHOLD({x.name},")]
+        assert block.count(" us against ") == len(x.values), x.name
 
 
 def test_error_strings():
@@ -228,9 +243,20 @@ class TestPlanner:
         assert fam((130, 65536)) == D and fam((63, 131072)) == D and fam((128, 65536), dtype=torch.bfloat16) == W
         for shape in [(300, 65536), (256, 65536), (512, 65536), (1024, 131072), (128, 131072), (2048, 32768)]:
             assert fam(shape, True) == D, shape
-        # rows of fewer than eight tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup
-        # each, except the backward of 512 rows and more with at least four such tiles
-        assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576)] for b in (False, True)] == [ST, D, ST, D, ST, ST]
+        # (the crossovers come from the generated table the library is compiled with)
+        T = nat.plan_thresholds()
+        # rows of few tiles of 4096 elements (and fewer than four of 8192) are left to one workgroup each, except
+        # the backward of enough rows with at least four such tiles
+        assert T["drift_min_small_tiles_per_row"] > 6 and 128 < T["drift_bwd_short_rows_min_rows"] <= 2048
+        short_bwd = lambda n: D if n >= T["drift_bwd_short_rows_min_rows"] else ST
+        assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576), (130, 16384)] for b in (False, True)] == \
+            [ST, short_bwd(2048), ST, short_bwd(768), ST, short_bwd(400), ST, short_bwd(130)]
+        n = T["drift_bwd_short_rows_min_rows"]
+        # (rows of seven such tiles: enough work in all for the rule on little work in many rows not to apply)
+        assert fam((n, 28672), True) == D and fam((n - 1, 28672), True) != D
+        k = T["drift_min_small_tiles_per_row"]
+        k += 1 - k % 2  # (an odd number of tiles of 4096 elements: not whole tiles of 8192)
+        assert fam((600, 4096 * k)) == D and fam((600, 4096 * (k - 2))) == W and fam((768, 4096 * (k - 2))) == ST
         # the backward of 16 to 127 rows with little work in all: teams that wait, with tiles of 16384 elements
         assert fam((96, 65536), True) == W and fam((24, 262144), True) == W
         assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
@@ -239,11 +265,13 @@ class TestPlanner:
         # 1024 rows of 16 tiles and more) or one workgroup per row; ragged rows one workgroup per row
         q = nat.plan(torch.empty(4096, 65536))
         assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 16, 256), q
-        assert fam((4096, 65536), True) == W and fam((2304, 131072), True) == ST and fam((4096, 65536 + 8)) == ST
+        m = T["drift_bwd_max_rows"]
+        assert 1024 <= m and fam((m, 65536), True) == D and fam((m + 256, 65536), True) == W
+        assert fam((m + 256, 131072), True) == ST and fam((4096, 65536 + 8)) == ST
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
         # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
-        assert slots((2304, 131072), True) == 8 and slots((256, 131072), True) == 1
+        assert slots((m + 256, 131072), True) == 8 and slots((256, 131072), True) == 1
         assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
@@ -255,7 +283,8 @@ class TestPlanner:
         assert [nat.plan(torch.empty(n, 65536 + 4))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
         assert nat.plan(torch.empty(300, 65536 + 4), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
         assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
-        assert fam((8, (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
+        assert fam((T["team_min_rows"], (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
+        assert fam((T["team_min_rows"] - 1, (1 << 20) + 4)) == nat.FAMILY_TILE      # fewer: look-back tiles
         assert fam((300, 65536), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
         assert fam((16, 1 << 20), dtype=torch.bfloat16) == nat.FAMILY_TEAM
         # 16-bit storage, forward: one or two very long rows in one team of the whole launch (tiles of 4096
