@@ -174,6 +174,10 @@ int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void*
  * linrec_fwd's.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
  * (two streams, two threads) race on it and must be serialised by the caller, and the array must not
  * be mixed with linrec_fwd's caller-owned workspaces in any other way than by calling this function.
+ * Where the table's kernel would need more than the array holds and no tuning is given, the call falls back
+ * to a kernel that needs less: one workgroup per row (rows on the unit-stride axis, at least a quarter as many as
+ * the device has compute units), or on a strided scan axis as many segments as fit, else one lane per row.
+ * LINREC_E_SCRATCH is what remains for a few very long rows, or when the caller's own tuning asks for more.
  * The array keeps the previous call's contents; nothing in it needs clearing between calls (its launch
  * counter tells old descriptors from new ones, and the completion counters end every launch at zero).
  * The first call on a device looks up the array's address there (hipGetSymbolAddress); make that call
@@ -183,6 +187,16 @@ int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void*
 int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t numseq,
                        int64_t seqlen, int64_t row_stride, int64_t elem_stride, int reverse,
                        const linrec_tuning_t* tuning, void* stream);
+/* The launch linrec_fwd_noalloc would make (its fallbacks included); LINREC_E_SCRATCH where it would turn the call down. */
+int linrec_plan_noalloc(int dtype, const void* any_input, int64_t numseq, int64_t seqlen, int64_t row_stride,
+                        int64_t elem_stride, int reverse, const linrec_tuning_t* tuning, linrec_plan_t* plan);
+/*
+ * Waits for another workgroup that hit the poll limit in linrec_fwd_noalloc launches on the current device so far
+ * (the second word of the static array's header; the results are right whatever the count).  Copies four words
+ * from the device, so it synchronises with it; -1 before the first linrec_fwd_noalloc call on the device.
+ * No counterpart in the reference.
+ */
+int linrec_noalloc_gave_up_count(void);
 
 /*
  * Batches of matrices whose scan axis is the strided one, e.g. (batch, time, channels) tensors
@@ -322,6 +336,23 @@ int linrec_stream_mix_f32(int reads, int writes, const float* src0, const float*
  */
 int linrec_stream_mix_order_f32(int reads, int writes, const float* src0, const float* src1, const float* src2,
                                 float* dst0, float* dst1, int64_t n, int hold_lo, int hold_bits, void* stream);
+
+/*
+ * Memory-only model of a drift launch: the same grid of persistent workgroups (one per compute unit) in teams
+ * of `team`, the same tiles of waves x slots x 256 floats in the same order, loads `ahead` tiles ahead and
+ * stores `late` steps late with one workgroup barrier per step - and neither a scan nor an exchange between
+ * workgroups.  Every tile's `reads` input streams are added up and stored to each of the `writes` outputs.
+ * What it takes is what the memory system gives that launch shape; a measuring instrument next to
+ * linrec_stream_mix_f32 (the same bytes by thousands of small workgroups in address order).
+ * Compiled: reads/writes 2/1 with waves x slots 16 x 2, 8 x 4, 16 x 1 and 3/2 with 16 x 1, 8 x 2; `ahead` 1 or 2,
+ * `late` 0 or 2 (LINREC_E_UNSUPPORTED otherwise).  `seqlen` a whole number of tiles, their number a multiple of `team`.
+ * stamps: NULL, or a device buffer of 2 x (workgroups) 64-bit words that receives every workgroup's wall clock
+ * (100 MHz) at its start and at its end; workgroups = min(numseq, compute units / team) x team.
+ * No counterpart in the reference.
+ */
+int linrec_launch_model_f32(int reads, int writes, const float* src0, const float* src1, const float* src2,
+                            float* dst0, float* dst1, int64_t numseq, int64_t seqlen, int waves, int slots,
+                            int team, int ahead, int late, unsigned long long* stamps, void* stream);
 
 /*
  * Batched matrix transpose on the device: src holds `batch` dense row-major matrices of rows x cols

@@ -84,6 +84,8 @@ def _declare(lib):
         "linrec_compute_units": (i32, []),
         "linrec_set_compute_units": (i32, [i32]),
         "linrec_fwd_noalloc": (i32, [i32, p, p, p, i64, i64, i64, i64, i32, tun, p]),
+        "linrec_noalloc_gave_up_count": (i32, []),
+        "linrec_plan_noalloc": (i32, [i32, p, i64, i64, i64, i64, i32, tun, plan]),
         "linrec_plan_threshold_count": (i32, []),
         "linrec_plan_threshold_name": (ctypes.c_char_p, [i32]),
         "linrec_plan_threshold_value": (i64, [i32]),
@@ -93,6 +95,7 @@ def _declare(lib):
         "linrec_copy_f32": (i32, [p, p, i64, p]),
         "linrec_stream_mix_f32": (i32, [i32, i32, p, p, p, p, p, i64, p]),
         "linrec_stream_mix_order_f32": (i32, [i32, i32, p, p, p, p, p, i64, i32, i32, p]),
+        "linrec_launch_model_f32": (i32, [i32, i32, p, p, p, p, p, i64, i64, i32, i32, i32, i32, i32, p, p]),
         "linrec_transpose": (i32, [i32, p, p, i64, i64, i64, p]),
         "linrec_fwd_batched": (i32, [i32, p, p, p, i64, i64, i64, i64, i64, i64, i32, p, sz, tun, p]),
         "linrec_bwd_batched": (i32, [i32, p, p, p, p, p, i64, i64, i64, i64, i64, i64, i32, p, sz, tun, p]),
@@ -215,28 +218,51 @@ def output_like(t, fake=False):
 
 
 # ---- look-back workspace, one per (device, stream) ---------------------------------------------
-_workspaces = collections.OrderedDict()  # least recently used first
+_workspaces = collections.OrderedDict()  # (device index, stream handle) -> buffer, least recently used first
+_ws_pinned = set()           # keys whose workspace a graph capture has been given: never dropped
+_ws_retired = []             # buffers a captured graph may still write to, outgrown since
+_ws_gave_up_of_dropped = {}  # device index -> waits that ran out, counted in workspaces since dropped
 _ws_lock = threading.Lock()
 _WS_MIN_BYTES = 1 << 20
 _WS_MAX_KEPT = 16  # (device, stream) pairs whose workspace is kept; a process rarely launches from more
 
 
+def _capturing():
+    """True while the current stream is being captured into a graph."""
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
 def workspace(device, stream_ptr, nbytes):
     """Zero-initialised scratch owned by the kernels' look-back chain.  Kept per stream because two
-    launches that overlap in time must not share descriptors; grown (and re-zeroed) on demand."""
+    launches that overlap in time must not share descriptors; grown (and re-zeroed) on demand.
+    A workspace handed out while its stream is being captured into a graph stays for good: the graph has
+    its address baked in and every replay writes descriptors there, so such a buffer is neither dropped with
+    the least recently used ones nor freed when a later launch on the stream needs a larger one."""
     key = (device.index, stream_ptr)
     with _ws_lock:
+        capturing = _capturing()
         ws = _workspaces.get(key)
         if ws is None or ws.numel() < nbytes:
             size = max(_WS_MIN_BYTES, 1 << (int(nbytes) - 1).bit_length())
+            if ws is not None and key in _ws_pinned:
+                _ws_retired.append(ws)
+                _ws_pinned.discard(key)
             ws = torch.zeros(size, dtype=torch.uint8, device=device)
             _workspaces[key] = ws
             # Streams come and go (their handles are even reused); the workspaces of the ones not
             # launched from for longest are dropped.  A dropped buffer goes back to torch's allocator,
             # which hands it out again in the order of the stream it was allocated on: the one its
             # kernels were queued on.
-            while len(_workspaces) > _WS_MAX_KEPT:
-                _workspaces.popitem(last=False)
+            if not capturing:
+                droppable = [k for k in _workspaces if k not in _ws_pinned and k != key]
+                while len(_workspaces) - len(_ws_pinned) > _WS_MAX_KEPT and droppable:
+                    old = droppable.pop(0)
+                    gone = _workspaces.pop(old)
+                    # (what it counted is kept; reading it synchronises, which is allowed outside a capture)
+                    if gone.is_cuda:
+                        _ws_gave_up_of_dropped[old[0]] = _ws_gave_up_of_dropped.get(old[0], 0) + int(gone[:16].view(torch.int32)[1].item())
+        if capturing:
+            _ws_pinned.add(key)
         _workspaces.move_to_end(key)
         return ws
 
@@ -453,11 +479,12 @@ def gave_up_count(device=None):
     """Waits for another workgroup that hit the poll limit, summed over this process's workspaces on
     `device` (synchronises).  The results are valid whatever the count (a wave whose wait runs out computes
     what it was waiting for from the row's own data); non-zero says that launches were slow."""
-    total = 0
+    want = None if device is None else torch.device(device).index
     with _ws_lock:
         items = list(_workspaces.items())
-    for (idx, _), ws in items:
-        if device is None or torch.device(device).index in (None, idx):
+        total = sum(n for idx, n in _ws_gave_up_of_dropped.items() if want in (None, idx))
+    for key, ws in items:
+        if want in (None, key[0]):
             total += int(ws[:16].view(torch.int32)[1].item())
     return total
 
@@ -584,3 +611,17 @@ def stream_mix(srcs, dsts, hold=(0, 0)):
         check(lib().linrec_stream_mix_order_f32(len(srcs), len(dsts), *ps, *pd, n, int(hold[0]), int(hold[1]),
                                                 torch.cuda.current_stream(ts[0].device).cuda_stream),
               "linrec_stream_mix_order_f32")
+
+
+def launch_model(srcs, dsts, shape, waves, slots, team, ahead=1, late=2, stamps=None):
+    """Memory-only model of a drift launch over dense float32 tensors of `shape` = (rows, length): the drift
+    kernels' workgroups, teams, tiles and order of accesses without scan or exchange (linrec_launch_model_f32).
+    `stamps`: int64 device tensor of 2 x workgroups words for every workgroup's start and end (100 MHz clock)."""
+    ts = list(srcs) + list(dsts)
+    assert ts and all(t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 and t.numel() == shape[0] * shape[1] for t in ts)
+    ps = [t.data_ptr() for t in srcs] + [None] * (3 - len(srcs))
+    pd = [t.data_ptr() for t in dsts] + [None] * (2 - len(dsts))
+    with torch.cuda.device(ts[0].device):
+        check(lib().linrec_launch_model_f32(len(srcs), len(dsts), *ps, *pd, shape[0], shape[1], waves, slots, team, ahead, late,
+                                            None if stamps is None else stamps.data_ptr(),
+                                            torch.cuda.current_stream(ts[0].device).cuda_stream), "linrec_launch_model_f32")

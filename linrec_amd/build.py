@@ -26,7 +26,7 @@ LIBNAME = "liblinrec_hip.so"
 DRIVER = "linrec_driver"
 SOURCES = ["linrec_capi.hip", "kernels_f32_rows.hip", "kernels_f32_teams.hip", "kernels_f32_walk.hip", "kernels_f32_cols.hip",
            "kernels_f16_rows.hip", "kernels_f16_cols.hip", "kernels_bf16_rows.hip", "kernels_bf16_cols.hip",
-           "linrec_host.cpp"]
+           "launch_model.hip", "linrec_host.cpp"]
 ARCH = "gfx950"
 
 FLAGS = [

@@ -350,6 +350,8 @@ int sweep_slots_for(const Problem& q, int fv) {
   const int64_t tiles_per_row = q.seqlen / (int64_t(8) * slots * 64 * fv);
   const int64_t least = slots == 8 ? least_tiles : kSweepMinTiles;
   if (tiles_per_row < least || sweep_team_size(tiles_per_row) < least) return 0;
+  // (a caller that can only give so much workspace is served by the kernels that need less)
+  if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) return 0;
   // 16-bit storage: measured gains only below the stream kernel's row counts (bf16 96 x 65536
   // 12.3 / 17.6 us against 17.5 / 24.7 us for one team per row, 160 x 262144 51 / 101 us against
   // 62 / 121 us; 1000 x 131072 backward 286 us against the stream kernel's 238 us).  Their backward
@@ -1461,6 +1463,51 @@ int linrec_fwd(int dtype, const void* inputs, const void* coeffs, void* outputs,
                   workspace_bytes, tuning, stream);
 }
 
+namespace {
+
+// The launch linrec_fwd_noalloc makes for `q` (q.workspace_cap set): the table's choice where the static array
+// holds its workspace, else - without a tuning of the caller's - a kernel that needs less: segments of a strided
+// scan axis as many as fit, or the kernels that need no workspace at all (one workgroup per row where the rows
+// give a quarter of the chip work; one lane per row or group of rows on a strided scan axis).  `effective`
+// receives the tuning to launch with (NULL for the table's choice).
+int noalloc_plan(const Problem& q, const linrec_tuning_t* tuning, linrec_plan_t* plan, linrec_tuning_t* storage,
+                 const linrec_tuning_t** effective) {
+  *effective = tuning;
+  const int rc = make_plan(q, tuning, plan);
+  if (rc != LINREC_OK) return rc;
+  if (plan->workspace_bytes <= q.workspace_cap) return LINREC_OK;
+  if (tuning) return LINREC_E_SCRATCH;  // (a caller's own tuning is not second-guessed)
+  auto fits = [&](const linrec_tuning_t& t) {
+    *storage = t;
+    return make_plan(q, storage, plan) == LINREC_OK && plan->family == t.family && plan->workspace_bytes <= q.workspace_cap;
+  };
+  bool found = false;
+  if (q.elem_stride == 1 || q.seqlen == 1) {
+    found = q.numseq * 4 >= q.cus && fits(linrec_tuning_t{LINREC_FAMILY_STREAM, 0, 0, -1, 0});
+  } else {
+    // (the maps of a segmented launch: two floats per row and segment, in the upper half of the workspace)
+    const int64_t segments = (int64_t(q.workspace_cap / 2) - 512) / (8 * q.numseq);
+    found = segments >= 2 && fits(linrec_tuning_t{LINREC_FAMILY_SEGMENT, 0, 0, -1, int32_t(std::min<int64_t>(segments, kSegmentMaxSegments))});
+    found = found || fits(linrec_tuning_t{LINREC_FAMILY_COLUMN, 0, 0, -1, 0}) || fits(linrec_tuning_t{LINREC_FAMILY_NAIVE, 0, 0, -1, 0});
+  }
+  if (!found) return LINREC_E_SCRATCH;
+  *effective = storage;
+  return LINREC_OK;
+}
+
+}  // namespace
+
+int linrec_plan_noalloc(int dtype, const void* any_input, int64_t numseq, int64_t seqlen, int64_t row_stride,
+                        int64_t elem_stride, int reverse, const linrec_tuning_t* tuning, linrec_plan_t* plan) {
+  if (!plan) return LINREC_E_INVALID;
+  if (dtype < LINREC_DTYPE_F32 || dtype > LINREC_DTYPE_BF16) return LINREC_E_UNSUPPORTED;
+  Problem q = forward_problem(dtype, any_input, any_input, any_input, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse);
+  q.workspace_cap = kStaticScratchBytes;
+  linrec_tuning_t storage;
+  const linrec_tuning_t* effective = nullptr;
+  return noalloc_plan(q, tuning, plan, &storage, &effective);
+}
+
 int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t numseq,
                        int64_t seqlen, int64_t row_stride, int64_t elem_stride, int reverse,
                        const linrec_tuning_t* tuning, void* stream) {
@@ -1470,13 +1517,12 @@ int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* 
   if (!inputs || !coeffs || !outputs) return LINREC_E_INVALID;
   // What the call needs follows from its arguments alone, so a call that needs more than the static
   // array holds is turned down before anything is enqueued.
-  // (kernels that would need more are left out of the choice where another one serves the call with less)
   Problem q = forward_problem(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse);
   q.workspace_cap = kStaticScratchBytes;
   linrec_plan_t plan;
-  const int rc = make_plan(q, tuning, &plan);
+  linrec_tuning_t storage;
+  const int rc = noalloc_plan(q, tuning, &plan, &storage, &tuning);
   if (rc != LINREC_OK) return rc;
-  if (plan.workspace_bytes > kStaticScratchBytes) return LINREC_E_SCRATCH;
   if (plan.workspace_bytes == 0)
     return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, nullptr, 0,
                     tuning, stream, kStaticScratchBytes);
@@ -1486,6 +1532,17 @@ int linrec_fwd_noalloc(int dtype, const void* inputs, const void* coeffs, void* 
   // The array's size is always passed whole: the split into counters and descriptors depends on it.
   return fwd_impl(dtype, inputs, coeffs, outputs, numseq, seqlen, row_stride, elem_stride, 0, 0, reverse, d->scratch_ptr,
                   kStaticScratchBytes, tuning, stream, kStaticScratchBytes);
+}
+
+int linrec_noalloc_gave_up_count(void) {
+  DeviceState* d = device_state();
+  if (!d || !d->scratch_ptr) return -1;
+  uint32_t header[4] = {0, 0, 0, 0};
+  if (hipMemcpy(header, d->scratch_ptr, sizeof(header), hipMemcpyDeviceToHost) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  return int(header[1] & 0x7fffffffu);
 }
 
 int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void* outputs, void* d_inputs,

@@ -11,12 +11,17 @@ one-thread-per-row kernel (eval/tune.py:98-102).
                               [--only TEXT] [--attrs] [--csv out.csv]
     python -m linrec_amd.tune --memory-probe [--shape 512 65536]
     python -m linrec_amd.tune --write-table [PATH]
+    python -m linrec_amd.tune --launch-model [--shape 512 65536]
 
 `--only TEXT` keeps the geometries whose label contains TEXT (one kernel under a profiler).
 `--write-table` measures the crossovers between the long-row kernels that the launch planner decides by (one
 sweep per threshold: the two kernels on either side, timed over a range of the quantity the rule is written in)
 and writes them as csrc/plan_thresholds.inc, the file the planner is compiled with - the counterpart of the
 dispatch table the reference's grid search writes (eval/tune.py:104-134).  Without PATH the file is printed.
+`--launch-model` times the memory-only model of the drift launch the planner makes for the shape (the same persistent
+workgroups, teams, tiles and order of accesses, no scan, no exchange), with its stores two steps late and at once
+and with one and two tiles of loads ahead, next to the scan kernels themselves and to the streaming kernel of
+thousands of small workgroups in address order; and when the model's workgroups, which all do the same work, end.
 `--memory-probe` times no scan at all: the memory-only kernel with a pass's mix of streams (2 in and 1 out,
 3 in and 2 out) over tensors of the given size, its 16 KiB blocks launched in address order and in orders
 that keep some address bits the same among the blocks in flight, which is what a launch with one
@@ -212,6 +217,60 @@ def memory_probe(shape, sets=3, iters=40, warmup=8, device="cuda:0"):
 
 
 
+def launch_model(shape, sets=3, iters=40, warmup=8, device="cuda:0"):
+    """Rows of dicts for fp32 tensors of `shape` whose planned launches are drift launches: per pass the scan kernel,
+    the memory-only model of its launch (variants of how far ahead it loads and how late it stores) and the streaming
+    kernel with the pass's mix of streams; for the model also when its workgroups end (us after the first start)."""
+    dev = torch.device(device)
+    n = shape[0] * shape[1]
+    srcs = [[torch.randn(shape, device=dev) for _ in range(3)] for _ in range(sets)]
+    dsts = [[torch.empty(shape, device=dev) for _ in range(2)] for _ in range(sets)]
+    for k in range(sets):
+        srcs[k][1].uniform_()  # coefficients in [0, 1)
+    names = nat.kernel_table()
+    rows = []
+    for is_bwd, nin, nout, bpe in ((False, 2, 1, 12), (True, 3, 2, 20)):
+        what = "backward" if is_bwd else "forward"
+        pl = nat.plan(srcs[0][0], False, is_bwd)
+        if pl["family"] != nat.FAMILY_DRIFT:
+            raise SystemExit(f"the planner's {what} launch for {shape} is not a drift launch ({names[pl['kernel_id']]})")
+        waves, slots, team = pl["waves"], pl["slots"], pl["tasks"]
+        grid = pl["grid"]
+        if is_bwd:
+            y = [nat.fwd(srcs[k][0], srcs[k][1]) for k in range(sets)]
+            t = _event_ms(lambda i: nat.bwd(srcs[i % sets][2], srcs[i % sets][1], y[i % sets], False,
+                                            out=(dsts[i % sets][0], dsts[i % sets][1])), iters, warmup)
+        else:
+            t = _event_ms(lambda i: nat.fwd(srcs[i % sets][0], srcs[i % sets][1], False, out=dsts[i % sets][0]), iters, warmup)
+
+        def row(label, ms, ends=None):
+            r = {"pass": what, "launch": label, "us": ms * 1e3, "GBps": bpe * n / ms / 1e6, "of_8_TBps": bpe * n / ms / 1e6 / 8000}
+            r.update({"first_end_us": float("nan"), "mean_end_us": float("nan"), "last_end_us": float("nan")} if ends is None else ends)
+            rows.append(r)
+
+        row(f"scan kernel {names[pl['kernel_id']]}, {grid} workgroups in teams of {team}", t)
+        kernel_ahead = 2 if (is_bwd and waves == 16 and slots == 1) else 1
+        variants = [(kernel_ahead, 2, "as the kernel"), (kernel_ahead, 0, "stores at once"), (3 - kernel_ahead, 2, "")]
+        for ahead, late, note in variants:
+            try:
+                nat.launch_model(srcs[0][:nin], dsts[0][:nout], shape, waves, slots, team, ahead, late)
+            except NotImplementedError:
+                continue
+            t = _event_ms(lambda i: nat.launch_model(srcs[i % sets][:nin], dsts[i % sets][:nout], shape, waves, slots, team, ahead, late),
+                          iters, warmup)
+            stamps = torch.zeros(2 * grid, dtype=torch.int64, device=dev)
+            nat.launch_model(srcs[0][:nin], dsts[0][:nout], shape, waves, slots, team, ahead, late, stamps)
+            st = stamps.view(grid, 2).cpu().double() * 0.01  # 100 MHz clock -> us
+            ends = st[:, 1] - st[:, 0].min()
+            row(f"memory-only model w{waves} s{slots} teams of {team}, {ahead} tile{'s' * (ahead > 1)} ahead, stores {late} steps late"
+                + (f" ({note})" if note else ""), t,
+                {"first_end_us": ends.min().item(), "mean_end_us": ends.mean().item(), "last_end_us": ends.max().item()})
+        t = _event_ms(lambda i: nat.stream_mix([a.view(-1) for a in srcs[i % sets][:nin]], [a.view(-1) for a in dsts[i % sets][:nout]]),
+                      iters, warmup)
+        row(f"streaming kernel, {n // 4096} workgroups of 4096 floats in address order", t)
+    return rows
+
+
 # ---- the planner's crossover thresholds ------------------------------------------------------------
 class Crossover:
     """One threshold of the planner: `name` in csrc/plan_thresholds.inc, the swept `values` of the quantity the
@@ -376,6 +435,8 @@ def main(argv=None):
     ap.add_argument("--only", default=None, metavar="TEXT", help="only the geometries whose label contains TEXT")
     ap.add_argument("--memory-probe", action="store_true",
                     help="time the memory-only kernel with address bits held among the blocks in flight instead")
+    ap.add_argument("--launch-model", action="store_true",
+                    help="time the memory-only model of the shape's drift launches next to the scan kernels instead")
     ap.add_argument("--attrs", action="store_true", help="print the register / LDS / scratch table instead")
     ap.add_argument("--write-table", nargs="?", const="-", default=None, metavar="PATH",
                     help="measure the planner's crossover thresholds and write csrc/plan_thresholds.inc (to PATH, or print it)")
@@ -392,6 +453,8 @@ def main(argv=None):
         rows = attrs_report()
     elif a.memory_probe:
         rows = memory_probe(tuple(a.shape))
+    elif a.launch_model:
+        rows = launch_model(tuple(a.shape))
     else:
         rows = sweep(tuple(a.shape), a.reverse, a.transposed, dtype=DTYPES[a.dtype], mixed_phase=a.mixed_phase, only=a.only)
     if not rows:

@@ -91,6 +91,27 @@ def test_write_table_measures_a_crossover_and_keeps_the_rest(tmp_path):
     assert text.count(" us against ") == len(x.values) and text.count("value kept") == len(cur) - 1
 
 
+def test_launch_model_reports_the_drift_launches_of_a_shape():
+    from linrec_amd import _native as nat, tune
+    rows = tune.launch_model((256, 65536), sets=1, iters=3, warmup=1)
+    for what in ("forward", "backward"):
+        mine = [r for r in rows if r["pass"] == what]
+        assert mine[0]["launch"].startswith("scan kernel drift_") and mine[-1]["launch"].startswith("streaming kernel")
+        models = [r for r in mine if r["launch"].startswith("memory-only model")]
+        assert len(models) >= 2 and "as the kernel" in models[0]["launch"]
+        assert all(r["us"] > 0 and 0 < r["first_end_us"] <= r["mean_end_us"] <= r["last_end_us"] for r in models)
+    # the model moves what it claims: every input tile added up into every output tile
+    x, c = torch.randn(16, 32768, device="cuda"), torch.randn(16, 32768, device="cuda")
+    out = torch.full_like(x, float("nan"))
+    nat.launch_model([x, c], [out], (16, 32768), 16, 2, 4, 1, 2)
+    assert torch.equal(out, x + c)
+    dy, o1, o2 = torch.randn_like(x), torch.full_like(x, float("nan")), torch.full_like(x, float("nan"))
+    nat.launch_model([x, c, dy], [o1, o2], (16, 32768), 16, 1, 8, 2, 2)
+    assert torch.equal(o1, x + c + dy) and torch.equal(o2, o1)
+    with pytest.raises(NotImplementedError):
+        nat.launch_model([x, c], [out], (16, 32768), 4, 4, 4, 1, 2)
+
+
 def test_memory_probe_reports_every_launch_order():
     from linrec_amd import tune
     rows = tune.memory_probe((64, 16384), sets=1, iters=3, warmup=1)

@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "linrec_hip.h")).read()
     declared = set(re.findall(r"^\s*(?:int|int64_t|size_t|const char\*|void)\s+(linrec_\w+)\s*\(", header, flags=re.M))
-    assert len(declared) == 32, declared
+    assert len(declared) == 35, declared
     lib = ctypes.CDLL(nat.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/linrec_hip.h but not exported"
@@ -139,6 +139,28 @@ def test_noalloc_entry_point_rejects_what_its_static_scratch_cannot_hold():
     assert need > limit
     assert lib.linrec_fwd_noalloc(0, fake, fake, fake, 1, n, n, 1, 0, None, None) == -5
     assert b"scratch" in lib.linrec_hip_error_string(-5)
+    # ... but where a kernel that needs less serves the problem, the call falls back to it: many long rows go to one
+    # workgroup per row, a strided scan axis to as many segments as the array holds maps for (or one lane per row)
+    def noalloc_plan(numseq, seqlen, row_stride, elem_stride, dtype=0, tuning=None):
+        pl = nat.Plan()
+        rc = lib.linrec_plan_noalloc(dtype, fake, numseq, seqlen, row_stride, elem_stride, 0,
+                                     ctypes.byref(tuning) if tuning else None, ctypes.byref(pl))
+        return rc, pl.asdict()
+    for rows, L in [(33000, 32768), (40001, 32768), (20001, 65536), (300, 8388608)]:
+        assert lib.linrec_workspace_bytes_dtype(0, rows, L, L, 1, 0, 0, None) > limit, (rows, L)
+        rc, pl = noalloc_plan(rows, L, L, 1)
+        # (300 rows: the 44 rows beyond one per compute unit in a second launch of teams, whose maps fit)
+        assert rc == 0 and pl["family"] == nat.FAMILY_STREAM and pl["workspace_bytes"] <= limit, (rows, L, rc, pl)
+        assert (pl["workspace_bytes"] == 0) == (pl["tail_rows"] == 0)
+    rc, pl = noalloc_plan(300, 65536, 65536, 1)  # (teams that exchange 2400 maps: the table's choice fits)
+    assert rc == 0 and pl["family"] == nat.FAMILY_DRIFT and 0 < pl["workspace_bytes"] <= limit
+    assert noalloc_plan(300, 8388608, 8388608, 1, tuning=nat.Tuning(nat.FAMILY_SWEEP))[0] == -5  # the caller's tuning stands
+    assert noalloc_plan(3, 1 << 30, 1 << 30, 1)[0] == -5  # too few rows for one workgroup each
+    rc, pl = noalloc_plan(3000, 200000, 1, 3000)  # transposed: segments, fewer than the table would take
+    assert lib.linrec_workspace_bytes_dtype(0, 3000, 200000, 1, 3000, 0, 0, None) > limit
+    assert rc == 0 and pl["family"] == nat.FAMILY_SEGMENT and pl["workspace_bytes"] <= limit and pl["tiles_per_row"] >= 2, pl
+    rc, pl = noalloc_plan(300000, 4096, 1, 300000)  # too many rows for two segments' maps: one lane per two rows
+    assert rc == 0 and pl["family"] == nat.FAMILY_COLUMN and pl["workspace_bytes"] == 0, pl
     # invalid arguments are reported as by linrec_fwd
     assert lib.linrec_fwd_noalloc(0, None, fake, fake, 4, 100000, 100000, 1, 0, None, None) == -1
     assert lib.linrec_fwd_noalloc(7, fake, fake, fake, 4, 100000, 100000, 1, 0, None, None) == -3
@@ -841,6 +863,18 @@ def test_caches_of_the_binding_stay_bounded(monkeypatch):
     assert made.count(nat._WS_MIN_BYTES) == 3 * nat._WS_MAX_KEPT  # stream 0 was allocated once
     ws = nat.workspace(dev, 0, nat._WS_MIN_BYTES + 1)  # growing replaces the buffer
     assert ws.numel() == 2 * nat._WS_MIN_BYTES and len(nat._workspaces) == nat._WS_MAX_KEPT
+    # a workspace handed out under graph capture is never dropped (the graph keeps writing to it), and is kept
+    # alive when a later launch on its stream needs a larger one
+    monkeypatch.setattr(nat, "_ws_pinned", set())
+    monkeypatch.setattr(nat, "_ws_retired", [])
+    monkeypatch.setattr(nat, "_capturing", lambda: True)
+    captured = nat.workspace(dev, 1000, 100)
+    monkeypatch.setattr(nat, "_capturing", lambda: False)
+    for stream in range(2000, 2000 + 2 * nat._WS_MAX_KEPT):
+        nat.workspace(dev, stream, 100)
+    assert nat._workspaces[(0, 1000)] is captured and len(nat._workspaces) == nat._WS_MAX_KEPT + 1
+    larger = nat.workspace(dev, 1000, nat._WS_MIN_BYTES + 1)
+    assert larger is not captured and any(w is captured for w in nat._ws_retired)
 
     monkeypatch.setattr(nat, "_need_cache", type(nat._need_cache)())
     monkeypatch.setattr(nat, "_NEED_CACHE_MAX", 8)

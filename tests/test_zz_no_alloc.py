@@ -65,6 +65,8 @@ def test_noalloc_forward_equals_forward_with_a_workspace_call_after_call():
     truth = oracle.fwd(x.cpu().numpy(), c.cpu().numpy(), False, dtype=np.float64)
     assert oracle.error_report(got.cpu().numpy(), truth)["normwise"] <= 1e-5
     assert nat.gave_up_count() == 0
+    # the waits of the launches on the static array are counted in its own header
+    assert nat.lib().linrec_noalloc_gave_up_count() == 0
 
 
 def test_noalloc_forward_of_16_bit_storage_and_kernels_without_scratch():
@@ -81,6 +83,48 @@ def test_noalloc_forward_of_16_bit_storage_and_kernels_without_scratch():
         want = nat.fwd(x, c)
         torch.cuda.synchronize()
         assert torch.equal(want, got), (dtype, shape)
+        # ... and against the float64 recurrence on the same rounded inputs: one rounding of the storage type
+        truth = oracle.fwd(x.float().cpu().numpy(), c.float().cpu().numpy(), False, dtype=np.float64)
+        ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 1e-5}[dtype]
+        assert oracle.error_report(got.float().cpu().numpy(), truth)["normwise"] <= ulp, (dtype, shape)
+    assert lib.linrec_noalloc_gave_up_count() == 0
+
+
+def test_noalloc_forward_under_graph_capture_and_replay():
+    """What the entry point is for: it is recorded into a HIP graph (after one call outside the capture, which looks
+    up the static array's address) and replayed, with the program's own launches and synchronisations in between,
+    and every replay must give the float64 recurrence's result."""
+    lib = nat.lib()
+    for shape, reverse in (((16, 131072), False), ((3, 40000), True)):
+        x, c = _pair(shape, 11)
+        lay = nat.row_layout(x)
+        out = torch.full_like(x, float("nan"))
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            assert lib.linrec_fwd_noalloc(0, x.data_ptr(), c.data_ptr(), out.data_ptr(), *lay, int(reverse), None,
+                                          side.cuda_stream) == 0  # warm-up on the capture stream
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.linrec_fwd_noalloc(0, x.data_ptr(), c.data_ptr(), out.data_ptr(), *lay, int(reverse), None,
+                                        torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+        for rep in range(3):
+            xs, cs = _pair(shape, 20 + rep)
+            x.copy_(xs)
+            c.copy_(cs)
+            out.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            truth = oracle.fwd(x.cpu().numpy(), c.cpu().numpy(), reverse, dtype=np.float64)
+            assert oracle.error_report(out.cpu().numpy(), truth)["normwise"] <= 1e-5, (shape, rep)
+            nat.fwd(xs, cs, reverse)  # (the program's own eager work between the replays)
+        del graph
+        assert torch.cuda.mem_get_info()[0] >= free_before - (64 << 20)  # (nothing the size of a workspace was allocated)
+    assert lib.linrec_noalloc_gave_up_count() == 0
 
 
 def test_noalloc_takes_another_kernel_where_the_usual_choice_needs_more_scratch_than_there_is():
@@ -107,11 +151,12 @@ def test_noalloc_takes_another_kernel_where_the_usual_choice_needs_more_scratch_
                                   ctypes.byref(t), torch.cuda.current_stream().cuda_stream) == -5
 
 
-def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row():
-    """20000 rows of 32768 elements: linrec_fwd takes teams that go from row to row, whose per-tile maps need more
-    than the 4 MiB there are; the entry point that allocates nothing walks every row with one workgroup instead."""
+@pytest.mark.parametrize("shape", [(20000, 32768), (33000, 32768)])
+def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row(shape):
+    """Tens of thousands of rows of 32768 elements: linrec_fwd takes teams that go from row to row, whose per-tile maps
+    need more than the 4 MiB there are; the entry point that allocates nothing walks every row with one workgroup."""
     lib = nat.lib()
-    x, c = _pair((20000, 32768), 6)
+    x, c = _pair(shape, 6)
     lay = nat.row_layout(x)
     need = lib.linrec_workspace_bytes_dtype(nat.DTYPES[x.dtype], *lay, 0, 0, None)
     assert nat.plan(x)["family"] == nat.FAMILY_DRIFT and need > (4 << 20)
@@ -122,7 +167,10 @@ def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row():
     want = nat.fwd(x, c)
     torch.cuda.synchronize()
     assert not torch.isnan(got).any()
-    rows = torch.tensor([0, 1, 255, 256, 9999, 19999], device=x.device)
+    pl = nat.Plan()
+    assert lib.linrec_plan_noalloc(0, x.data_ptr(), *lay, 0, None, ctypes.byref(pl)) == 0
+    assert pl.family == nat.FAMILY_STREAM and pl.workspace_bytes == 0
+    rows = torch.tensor([0, 1, 255, 256, 9999, shape[0] - 1], device=x.device)
     truth = oracle.fwd(x.index_select(0, rows).cpu().numpy(), c.index_select(0, rows).cpu().numpy(), False, dtype=np.float64)
     assert oracle.error_report(got.index_select(0, rows).cpu().numpy(), truth)["normwise"] <= 1e-5
     assert oracle.error_report(want.index_select(0, rows).cpu().numpy(), truth)["normwise"] <= 1e-5
