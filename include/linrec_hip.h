@@ -163,6 +163,30 @@ int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void*
                void* stream);
 
 /*
+ * linrec_fwd / linrec_bwd with the arguments in one block of memory, for bindings whose cost per argument
+ * counts (a ctypes call marshals every argument; on a 64 x 4096 tensor, whose kernel takes 3 us, the
+ * binding then spends more time than the device).  The caller keeps a linrec_call_t per kind of call and only
+ * rewrites the pointers.  Forward: in0 = inputs, out0 = outputs; backward: in0 = d_outputs, aux = outputs,
+ * out0 = d_inputs, out1 = d_coeffs.  Same results and error codes as linrec_fwd / linrec_bwd with no tuning.
+ * The counterpart of the reference's one pybind call per pass (linrec/impl/cuda/extension.cpp:61-67).
+ */
+typedef struct linrec_call {
+  int32_t dtype;    /* LINREC_DTYPE_* */
+  int32_t reverse;
+  int64_t numseq, seqlen, row_stride, elem_stride;
+  const void* in0;
+  const void* coef;
+  const void* aux;
+  void* out0;
+  void* out1;
+  void* workspace;
+  uint64_t workspace_bytes;
+  void* stream;
+} linrec_call_t;
+int linrec_fwd_call(const linrec_call_t* call);
+int linrec_bwd_call(const linrec_call_t* call);
+
+/*
  * linrec_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc): the same call without the workspace arguments.
  * It has no counterpart in the reference, whose launcher allocates its result itself

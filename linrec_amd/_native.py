@@ -61,6 +61,15 @@ class Plan(ctypes.Structure):
         return {name: getattr(self, name) for name, _ in self._fields_}
 
 
+class Call(ctypes.Structure):
+    """linrec_call_t: the arguments of linrec_fwd_call / linrec_bwd_call in one block of memory."""
+    _fields_ = [("dtype", ctypes.c_int32), ("reverse", ctypes.c_int32), ("numseq", ctypes.c_int64),
+                ("seqlen", ctypes.c_int64), ("row_stride", ctypes.c_int64), ("elem_stride", ctypes.c_int64),
+                ("in0", ctypes.c_void_p), ("coef", ctypes.c_void_p), ("aux", ctypes.c_void_p),
+                ("out0", ctypes.c_void_p), ("out1", ctypes.c_void_p), ("workspace", ctypes.c_void_p),
+                ("workspace_bytes", ctypes.c_uint64), ("stream", ctypes.c_void_p)]
+
+
 _lib = None
 _lib_lock = threading.Lock()
 
@@ -84,6 +93,8 @@ def _declare(lib):
         "linrec_compute_units": (i32, []),
         "linrec_set_compute_units": (i32, [i32]),
         "linrec_fwd_noalloc": (i32, [i32, p, p, p, i64, i64, i64, i64, i32, tun, p]),
+        "linrec_fwd_call": (i32, [ctypes.POINTER(Call)]),
+        "linrec_bwd_call": (i32, [ctypes.POINTER(Call)]),
         "linrec_noalloc_gave_up_count": (i32, []),
         "linrec_plan_noalloc": (i32, [i32, p, i64, i64, i64, i64, i32, tun, plan]),
         "linrec_plan_threshold_count": (i32, []),
@@ -352,10 +363,12 @@ _NEED_CACHE_MAX = 1024
 
 def set_compute_units(cus):
     """Overrides the compute-unit count the planner sizes its launches by (0: ask the device again) and
-    forgets the workspace sizes remembered for the count in force before.  Returns the previous override."""
+    forgets the workspace sizes remembered for the count in force before (those of other threads' repeat calls
+    are forgotten when those threads next look: the override is a testing aid).  Returns the previous override."""
     old = lib().linrec_set_compute_units(cus)
     if cus >= 0:
         _need_cache.clear()
+        _repeat_table().clear()
     return old
 
 
@@ -507,9 +520,130 @@ def _few_rows_on_strided_axis(t, lay, tuning):
     return _RELAYOUT_UNIT_ROW_STRIDE or (lay[2] != 1 and lay[0] != 1)
 
 
+# ---- repeat calls ------------------------------------------------------------------------------
+# A call on device tensors whose sizes, strides, types and devices have been seen before (on this thread) skips
+# everything that only depends on those: validation, the layout, the workspace size; what is left is the
+# pointers (which must be 16-byte aligned, as the results then are), the stream and one library call that takes
+# its arguments in one block of memory.  On a 64 x 4096 tensor, whose kernel takes 3 us, this halves the time
+# the host needs per launch.  Everything else takes the general path below.
+_repeat = threading.local()
+_REPEAT_MAX = 256
+
+
+def _repeat_table():
+    table = getattr(_repeat, "table", None)
+    if table is None:
+        table = _repeat.table = {}
+    return table
+
+
+def _remember(table, key, lay, t, is_bwd, reverse):
+    """What a repeat of the call `key` needs: (Call, reference to it, workspace bytes), or None if calls of
+    this kind take the general path."""
+    entry = None
+    if lay is not None:
+        call = Call(dtype=DTYPES[t.dtype], reverse=int(bool(reverse)), numseq=lay[0], seqlen=lay[1], row_stride=lay[2],
+                    elem_stride=lay[3])
+        need = lib().linrec_workspace_bytes_dtype(DTYPES[t.dtype], *lay, 0, int(is_bwd), None)
+        entry = (call, ctypes.byref(call), int(need))
+    if len(table) >= _REPEAT_MAX:
+        table.clear()
+    table[key] = entry
+    return entry
+
+
+def _repeat_launch(entry, fn, t, what):
+    call, ref, need = entry
+    idx = t.device.index
+    if torch.cuda.current_device() == idx:
+        stream = _raw_stream(idx)
+        if need:
+            ws = workspace(t.device, stream, need)
+            call.workspace, call.workspace_bytes = ws.data_ptr(), ws.numel()
+        call.stream = stream
+        rc = fn(ref)
+    else:
+        with torch.cuda.device(idx):
+            stream = _raw_stream(idx)
+            if need:
+                ws = workspace(t.device, stream, need)
+                call.workspace, call.workspace_bytes = ws.data_ptr(), ws.numel()
+            call.stream = stream
+            rc = fn(ref)
+    if rc:
+        check(rc, what)
+
+
+def _plain_rows(t, lay, *same):
+    """The layout if a call on `t` (and tensors `same`, which must lie in memory like it) can be repeated
+    from remembered arguments, else None."""
+    if lay is None or not t.is_cuda or t.dtype not in DTYPES or not t.numel() or _few_rows_on_strided_axis(t, lay, None):
+        return None
+    return lay if _same_layout(t, *same) else None
+
+
 def fwd(inputs, coeffs, reverse=False, tuning=None, out=None):
     """outputs = linrec(inputs, coeffs) over the last dim (linrec/impl/cuda/linrec_pipe.cu:16-92).
     `out`, if given, must have the layout the result would be allocated with."""
+    if tuning is None and inputs.is_cuda:
+        shape, stride = inputs.shape, inputs.stride()
+        key = (inputs.dtype, inputs.device, shape, stride, coeffs.dtype, coeffs.device, coeffs.shape, coeffs.stride(), reverse)
+        table = _repeat_table()
+        entry = table.get(key, False)
+        if entry is False:
+            _validate(inputs, coeffs, names=("inputs", "coeffs"))
+            entry = _remember(table, key, _plain_rows(inputs, row_layout(inputs), coeffs), inputs, False, reverse)
+        if entry is not None:
+            px, pc = inputs.data_ptr(), coeffs.data_ptr()
+            if not (px | pc) & 15:
+                if out is None:
+                    res = torch.empty_strided(shape, stride, dtype=inputs.dtype, device=inputs.device)
+                elif out.shape == shape and out.stride() == stride and out.dtype == inputs.dtype and out.device == inputs.device:
+                    res = out
+                else:
+                    raise RuntimeError("linrec: `out` does not have the layout of the (canonicalised) inputs")
+                po = res.data_ptr()
+                if not po & 15:
+                    call = entry[0]
+                    call.in0, call.coef, call.out0 = px, pc, po
+                    _repeat_launch(entry, lib().linrec_fwd_call, inputs, "linrec_fwd")
+                    return res
+    return _fwd_general(inputs, coeffs, reverse, tuning, out)
+
+
+def bwd(d_outputs, coeffs, outputs, reverse=False, tuning=None, out=None):
+    """(d_inputs, d_coeffs) (linrec/impl/cuda/linrec_pipe.cu:96-174).  The three tensors are brought
+    to one memory layout first (the reference instead requires equal strides, linrec_pipe.cu:98)."""
+    if tuning is None and outputs.is_cuda:
+        shape, stride = outputs.shape, outputs.stride()
+        key = (outputs.dtype, outputs.device, shape, stride, coeffs.dtype, coeffs.device, coeffs.shape, coeffs.stride(),
+               d_outputs.dtype, d_outputs.device, d_outputs.shape, d_outputs.stride(), reverse, True)
+        table = _repeat_table()
+        entry = table.get(key, False)
+        if entry is False:
+            _validate(outputs, coeffs, d_outputs, names=("outputs", "coeffs", "d_outputs"))
+            entry = _remember(table, key, _plain_rows(outputs, row_layout(outputs), coeffs, d_outputs), outputs, True, reverse)
+        if entry is not None:
+            pd, pc, py = d_outputs.data_ptr(), coeffs.data_ptr(), outputs.data_ptr()
+            if not (pd | pc | py) & 15:
+                if out is None:
+                    dx = torch.empty_strided(shape, stride, dtype=outputs.dtype, device=outputs.device)
+                    dc = torch.empty_strided(shape, stride, dtype=outputs.dtype, device=outputs.device)
+                else:
+                    dx, dc = out
+                    if not (_same_layout(outputs, dx, dc) and dx.dtype == outputs.dtype == dc.dtype
+                            and dx.device == outputs.device == dc.device):
+                        raise RuntimeError("linrec: `out` tensors do not have the layout of the (canonicalised) outputs")
+                p0, p1 = dx.data_ptr(), dc.data_ptr()
+                if not (p0 | p1) & 15:
+                    call = entry[0]
+                    call.in0, call.coef, call.aux, call.out0, call.out1 = pd, pc, py, p0, p1
+                    _repeat_launch(entry, lib().linrec_bwd_call, outputs, "linrec_bwd")
+                    return dx, dc
+    return _bwd_general(d_outputs, coeffs, outputs, reverse, tuning, out)
+
+
+def _fwd_general(inputs, coeffs, reverse=False, tuning=None, out=None):
     _validate(inputs, coeffs, names=("inputs", "coeffs"))
     if not inputs.is_cuda and inputs.dtype in (torch.float16, torch.bfloat16):
         # host tensors in a 16-bit type: fp32 arithmetic, one rounding at the end, as on the device
@@ -535,9 +669,7 @@ def fwd(inputs, coeffs, reverse=False, tuning=None, out=None):
     return outputs
 
 
-def bwd(d_outputs, coeffs, outputs, reverse=False, tuning=None, out=None):
-    """(d_inputs, d_coeffs) (linrec/impl/cuda/linrec_pipe.cu:96-174).  The three tensors are brought
-    to one memory layout first (the reference instead requires equal strides, linrec_pipe.cu:98)."""
+def _bwd_general(d_outputs, coeffs, outputs, reverse=False, tuning=None, out=None):
     _validate(outputs, coeffs, d_outputs, names=("outputs", "coeffs", "d_outputs"))
     if not outputs.is_cuda and outputs.dtype in (torch.float16, torch.bfloat16):
         dx, dc = bwd(d_outputs.float(), coeffs.float(), outputs.float(), reverse)

@@ -1553,6 +1553,18 @@ int linrec_bwd(int dtype, const void* d_outputs, const void* coeffs, const void*
                   reverse, workspace, workspace_bytes, tuning, stream);
 }
 
+int linrec_fwd_call(const linrec_call_t* c) {
+  if (!c) return LINREC_E_INVALID;
+  return fwd_impl(c->dtype, c->in0, c->coef, c->out0, c->numseq, c->seqlen, c->row_stride, c->elem_stride, 0, 0, c->reverse,
+                  c->workspace, size_t(c->workspace_bytes), nullptr, c->stream);
+}
+
+int linrec_bwd_call(const linrec_call_t* c) {
+  if (!c) return LINREC_E_INVALID;
+  return bwd_impl(c->dtype, c->in0, c->coef, c->aux, c->out0, c->out1, c->numseq, c->seqlen, c->row_stride, c->elem_stride, 0,
+                  0, c->reverse, c->workspace, size_t(c->workspace_bytes), nullptr, c->stream);
+}
+
 int linrec_fwd_batched(int dtype, const void* inputs, const void* coeffs, void* outputs, int64_t batches,
                        int64_t rows_per_batch, int64_t seqlen, int64_t batch_stride, int64_t row_stride,
                        int64_t elem_stride, int reverse, void* workspace, size_t workspace_bytes,

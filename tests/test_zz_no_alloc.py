@@ -151,7 +151,7 @@ def test_noalloc_takes_another_kernel_where_the_usual_choice_needs_more_scratch_
                                   ctypes.byref(t), torch.cuda.current_stream().cuda_stream) == -5
 
 
-@pytest.mark.parametrize("shape", [(20000, 32768), (33000, 32768)])
+@pytest.mark.parametrize("shape", [(33000, 32768), (20001, 65536)])
 def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row(shape):
     """Tens of thousands of rows of 32768 elements: linrec_fwd takes teams that go from row to row, whose per-tile maps
     need more than the 4 MiB there are; the entry point that allocates nothing walks every row with one workgroup."""
@@ -159,7 +159,7 @@ def test_noalloc_serves_many_long_rows_with_one_workgroup_per_row(shape):
     x, c = _pair(shape, 6)
     lay = nat.row_layout(x)
     need = lib.linrec_workspace_bytes_dtype(nat.DTYPES[x.dtype], *lay, 0, 0, None)
-    assert nat.plan(x)["family"] == nat.FAMILY_DRIFT and need > (4 << 20)
+    assert nat.plan(x)["family"] in (nat.FAMILY_DRIFT, nat.FAMILY_SWEEP) and need > (4 << 20)
     got = torch.full_like(x, float("nan"))
     rc = lib.linrec_fwd_noalloc(nat.DTYPES[x.dtype], x.data_ptr(), c.data_ptr(), got.data_ptr(), *lay, 0, None,
                                 torch.cuda.current_stream().cuda_stream)
