@@ -76,7 +76,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   constexpr bool NEED_Y = MODE == 1;
   const int ksteps = (L + STEP - 1) / STEP;              // steps of the whole row
   const int own = j < ksteps ? (ksteps - j + M - 1) / M : 0;  // steps of this workgroup: j, j + M, ...
-  const uint32_t seq = __hip_atomic_load(&ch.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint32_t seq = load_seq_through_caches(ch.ws);
   const uint32_t want = (seq << 2) | STATUS_AGGREGATE;
   if (threadIdx.x < 4) sh_fail[threadIdx.x] = -1;
   __syncthreads();

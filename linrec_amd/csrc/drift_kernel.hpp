@@ -66,9 +66,10 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   const long long my_rows = team < p.numseq ? (p.numseq - team + teams - 1) / teams : 0;
   const int items = int(my_rows * per_row);
 
-  const uint32_t seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (threadIdx.x < 4) sh_fail[threadIdx.x] = 0;
-  __syncthreads();
+  // (read through the scalar cache: it arrives beside the first tile's loads instead of holding them up, which an
+  // agent-scope load did for a memory round trip at the start of every launch)
+  const uint32_t seq = load_seq_through_caches(p.ws);
+  if (threadIdx.x < 4) sh_fail[threadIdx.x] = 0;  // (every reader has passed a step's barrier first)
   const RowView rv = make_row_view<VEC>(0, 0, p.seqlen);
 
   struct Item {

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(64 * NW) void sweep_kernel(TileArgs p) {
 
   uint32_t seq = 0;
   uint32_t leaf_count = 0;
-  if (wave == 0) seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (wave == 0) seq = load_seq_through_caches(p.ws);
 
   // all rows look alike: aligned, seqlen / VEC full slots
   const RowView rv = make_row_view<VEC>(0, 0, p.seqlen);

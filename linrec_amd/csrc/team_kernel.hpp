@@ -70,7 +70,7 @@ __global__ __launch_bounds__(64 * NW) void team_kernel(TileArgs p) {
 
   uint32_t seq = 0;
   uint32_t leaf_count = 0;
-  if (wave == 0) seq = __hip_atomic_load(&p.ws->seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (wave == 0) seq = load_seq_through_caches(p.ws);
 
   const long long row_off = row * p.row_stride;
   const RowView rv = make_row_view<VEC>(p.base_mis, row_off, p.seqlen);

@@ -55,12 +55,12 @@ struct TileArgs {
 #endif
 };
 
-// The sequence number of a launch of many tiles, read through the caches.  The word only changes when the
-// launch's last tile is done, by which time every tile has read it, and a launch starts with the caches written
-// back and invalidated, so what it reads is what the launch before it left.  An agent-scope load goes to memory
-// every time, where thousands of tiles asking for the one address queue up: 512 x 65536 in look-back tiles of 4096
-// elements takes 109 us with it and 79 us with this.  (The kernels of a few hundred workgroups keep the
-// agent-scope load.)
+// The sequence number of a launch, read through the caches.  The word only changes when the launch's last
+// workgroup is done, by which time every workgroup has read it, and a launch starts with the caches written back
+// and invalidated, so what it reads is what the launch before it left.  An agent-scope load goes to memory every
+// time: thousands of tiles asking for the one address queue up there (512 x 65536 in look-back tiles of 4096
+// elements takes 109 us with it and 79 us with this), and a persistent workgroup that waits for it before its
+// first loads starts a memory round trip late.
 __device__ __forceinline__ uint32_t load_seq_through_caches(const CarryHeader* ws) { return ws->seq; }
 
 __device__ __forceinline__ uint64_t pack_desc(uint32_t flag, float v) {

@@ -661,15 +661,20 @@ def test_little_work_in_many_rows_goes_to_small_teams_with_the_largest_tiles(nat
 @pytest.mark.parametrize("reverse", [False, True])
 def test_more_than_2048_rows_of_whole_tiles_run_forward_in_teams(nat, reverse):
     """Beyond 2048 rows the forward still goes to the teams whose tiles are stored two steps late (tiles of 4096
-    elements, 16 waves), the backward to the teams that wait or to one workgroup per row."""
+    elements, 16 waves) where a row has enough such tiles (the planner's generated threshold), the backward to them
+    as well up to its own threshold, else to the teams that wait or to one workgroup per row."""
     dev = torch.device("cuda:0")
-    for n, L, team in [(2100, 32768, 8), (2200, 4096 * 9, 9)]:
+    k = nat.plan_thresholds()["drift_min_small_tiles_per_row"]
+    k += 1 - k % 2  # (odd: whole tiles of 4096 elements but not of 8192)
+    for n, L, team in [(2100, 4096 * (k + 1), k + 1), (2200, 4096 * k, k)]:
         g = torch.Generator().manual_seed(n)
         x, c, dy = (torch.randn(n, L, generator=g), torch.rand(n, L, generator=g), torch.randn(n, L, generator=g))
         xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
         plan = nat.plan(xd, reverse)
         assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == (nat.FAMILY_DRIFT, 16, 1, team), plan
-        assert nat.plan(xd, reverse, True)["family"] in (nat.FAMILY_SWEEP, nat.FAMILY_STREAM)
+        bwd_family = nat.plan(xd, reverse, True)["family"]
+        assert bwd_family == (nat.FAMILY_DRIFT if n <= nat.plan_thresholds()["drift_bwd_max_rows"] else bwd_family)
+        assert bwd_family in (nat.FAMILY_SWEEP, nat.FAMILY_STREAM, nat.FAMILY_DRIFT)
         y = nat.fwd(xd, cd, reverse)
         dx, dc = nat.bwd(dyd, cd, y, reverse)
         torch.cuda.synchronize()
