@@ -91,15 +91,21 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     return make_row_ptrs<T, MODE>(p.in0, p.coef, p.aux, p.out0, p.out1, (long long)row * p.row_stride, 0);
   };
 
+  // 16-bit storage: the tiles whose loads are in flight, and a pending tile's saved outputs, stay in the storage
+  // type until their step comes (half the registers, and no conversion that would have to wait for the loads in
+  // the step that issues them).
+  constexpr bool PACKED = !std::is_same_v<T, float>;
+  using Loaded = std::conditional_t<PACKED, TilePacked<T, S, VEC, MODE>, TileData<S, VEC, MODE>>;
   // A tile that has been scanned and not stored yet.
   struct Pending {
-    TileData<S, VEC, MODE> d;  // (what the store still needs of it: the saved outputs, backward)
+    Loaded d;    // (what the store still needs of it: the saved outputs, backward)
+    float edge;  // 16-bit storage, backward: the saved output after the wave's last, wave-uniform (a scalar register)
     TileScan<S, VEC> r;
     Affine before;  // the waves in front of this one
     Affine total;   // the whole tile's map
     Item it;
   };
-  TileData<S, VEC, MODE> D[3];  // tile n lies in D[n % 3]
+  Loaded D[3];  // tile n lies in D[n % 3]
   Item DI[3];
   Pending P[3];                 // and becomes P[n % 3]
 
@@ -226,6 +232,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       }
     }
     own_out = t == 0 ? q.total.b : fmaf(carry_in, q.total.a, q.total.b);
+    if constexpr (PACKED) own_out = read_lane(own_out, 0);  // (wave-uniform: a scalar register, where vector registers are short)
     return carry_in;
   };
   auto store_pending = [&](const Pending& q, float tile_in) {
@@ -239,12 +246,20 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       has_entry = true;
       entry = q.before.b;
     }
-    tile_apply_store<S, VEC, MODE, DESC, true>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS, lane,
-                                               has_entry, entry);
+    if constexpr (PACKED) {
+      tile_apply_store_packed<S, VEC, MODE, DESC>(q.d.ys, q.edge, q.r, ptrs_of(q.it.row), rv,
+                                                  t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+    } else {
+      tile_apply_store<S, VEC, MODE, DESC, true>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS,
+                                                 lane, has_entry, entry);
+    }
   };
-  auto load_next = [&](TileData<S, VEC, MODE>& d, Item& it) {
+  auto load_next = [&](Loaded& d, Item& it) {
     it = next_item();
-    tile_load<S, VEC, MODE, DESC, true>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane, false);
+    if constexpr (PACKED)
+      tile_load_packed<S, VEC, MODE, DESC>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane);
+    else
+      tile_load<S, VEC, MODE, DESC, true>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane, false);
   };
 
   // Step n, n % 3 == PH: tile n lies in D[PH]; P[(PH + 1) % 3] is tile n-2, stored in this step.
@@ -255,7 +270,15 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     if (n >= 2 && (wide || wave == 0)) ask(P[OLD].it, w0, w1);
     __builtin_amdgcn_sched_barrier(0);
     if (prefetch) load_next(D[LD], DI[LD]);
-    TileData<S, VEC, MODE>& d = D[PH];
+    TileData<S, VEC, MODE> unpacked;
+    TileData<S, VEC, MODE>& d = [&]() -> TileData<S, VEC, MODE>& {
+      if constexpr (PACKED) {
+        tile_unpack<S, VEC, MODE, DESC>(D[PH], unpacked);
+        return unpacked;
+      } else {
+        return D[PH];
+      }
+    }();
     const Item it = DI[PH];
     if constexpr (MODE == MODE_FWD) {
       if (it.t == 0 && wave == 0 && lane == 0) d.cs[0][0] = 0.0f;  // the row's first coefficient takes no part
@@ -266,6 +289,21 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       // a slot's map from the wave's entry value to the slot's is folded into the elements' maps, which leaves
       // a pending tile two values per element and nothing per slot (16 waves have 128 registers each); nothing
       // enters a row's first wave, whose factors are therefore zero and never meet a product that overflowed
+      const bool nothing_enters = it.t == 0 && wave == 0;
+#pragma unroll
+      for (int j = 0; j < S; ++j) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
+          now.r.pa[j][i] = nothing_enters ? 0.0f : now.r.pa[j][i] * now.r.ex_a[j];
+        }
+        now.r.ex_a[j] = 1.0f;
+        now.r.ex_b[j] = 0.0f;
+      }
+    }
+    if constexpr (MODE == MODE_BWD && PACKED) {
+      // 16-bit storage: the same folding in the backward (whose first factor of a slot is one before it), one
+      // register less for each of the three tiles in the works
       const bool nothing_enters = it.t == 0 && wave == 0;
 #pragma unroll
       for (int j = 0; j < S; ++j) {
@@ -297,7 +335,10 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       const float tile_in = combine(P[OLD], par, n);
       store_pending(P[OLD], tile_in);
     }
-    if constexpr (MODE == MODE_BWD) now.d = d;
+    if constexpr (MODE == MODE_BWD) {
+      now.d = D[PH];
+      if constexpr (PACKED) now.edge = read_lane(d.y_edge, 63);  // (only lane 63 holds it, only lane 63 uses it)
+    }
     now.it = it;
   };
   // The last tile lies in P[A] and the one before it in P[(A + 2) % 3]: nothing left to overlap with, so

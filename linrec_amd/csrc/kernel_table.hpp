@@ -64,10 +64,12 @@ KernelGroup kernels_bf16_cols();
 // only 48 KB (one after the other in one process, us, against 8 waves of two slots with one tile ahead, which one
 // tile ahead in 16 waves had beaten by 1 to 4 %: 512 x 65536 112.4 against 117.5, 300 x 65536 68.3 against 71.2,
 // 16 x 1048576 60.1 against 63.6, 1 x 33554432 111.6 against 124.5); the forward gains nothing from it.
-#define DRIFT_TILES_AHEAD(NW, S, MODE) ((NW) == 16 && (S) == 1 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
+// (16-bit storage, eight elements per slot: a second tile does not fit the backward's registers and brings the
+// forward nothing: bf16 512 x 65536 40.2 against 40.4 us, 16 x 1048576 25.2 against 25.0)
+#define DRIFT_TILES_AHEAD(NW, S, VEC, MODE) ((NW) == 16 && (S) == 1 && (VEC) == 4 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, VEC, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
@@ -160,12 +162,13 @@ KernelGroup kernels_bf16_cols();
 
 // The 16-bit storage types get the geometries the planner picks for them (their register tiles are
 // twice as wide as fp32's, so two slots of eight elements per lane is the rule; the forward team
-// kernel, which keeps its prefetched tile packed, also comes with four).
+// kernel also comes with four, and the drift kernels, which keep three tiles in the works, with one).
 #define HALF_ROW_KERNELS(TY)                                                                    \
   TILE_(TY, 1, 1, 8, 0), TILE_(TY, 2, 1, 8, 0), TILE_(TY, 4, 1, 8, 0), TILE_(TY, 4, 2, 8, 0),   \
   TILE_(TY, 8, 2, 8, 0), TILE_(TY, 16, 2, 8, 0), TILE_(TY, 4, 2, 8, 1), TILE_(TY, 8, 4, 8, 1),  \
   TILE_(TY, 4, 4, 1, 0), TILE_(TY, 4, 4, 1, 1), STREAM_(TY, 8, 2, 8), TEAM_(TY, 8, 2, 8),       \
-  TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8)
+  TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8),                            \
+  DRIFT_FWD_(TY, 16, 1, 8), DRIFT_BWD_(TY, 16, 1, 8)
 #define HALF_COLUMN_KERNELS(TY)                                                                 \
   GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
   COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16), \

@@ -259,18 +259,41 @@ bool little_work_in_many_rows(const Problem& q) {
 // The largest team a drift kernel of this geometry serves: a lane of a wave per team mate, in every wave - except
 // 16 waves of two slots, compiled for one collecting wave.
 int64_t drift_max_team(int waves, int slots) { return waves == 16 && slots == 2 ? 64 : int64_t(64) * waves; }
+// 16-bit storage: tiles of 8192 elements in 16 waves (tiles in flight stay in the storage type, so a lane's eight
+// elements of a slot cost what four fp32 elements do), or of 4096 in 8 waves, forward only, for one or two rows that
+// are not whole tiles of 8192.  Returns 2 or 1 accordingly, 0 for "not a drift case".
+// The backward wins wherever the fp32 one does (bf16, us, against the table's choice before: 512 x 65536 56.9
+// against 63.8 for one workgroup per row, 300 x 65536 36.3 against 44.0, 2048 x 32768 110.7 against 121.4, 1024 x
+// 131072 220.7 against 246.9; 16 x 1048576 31.5 against 41.8 for one team per row, 64 x 524288 57.2 against 70.5;
+// 1 x 33554432 59.7 against 83.9 for look-back tiles, 1 x 4194304 16.1 against 18.7, 24 x 262144 15.9 against 18.0;
+// but 1 x 1048576 16.6 against 15.1).  The forward, whose step moves 48 KB, only where the rows are too few for one
+// workgroup per row (1 x 33554432 43.4 against 61.3 us in tiles of 4096, 3 x 4194304 21.1 against 27.6 for one team
+// per row, 64 x 524288 40.7 against 45.2, 96 x 262144 30.9 against 32.9, 16 x 1048576 25.2 against 25.5; rows of 32
+// tiles and more up to 255 of them: 128 x 262144 39.2 against 41.1, 160 x 262144 47.9 against 51.4; but 128 x 65536
+// 14.5 against 12.9, 200 x 65536 19.8 against 16.4, 512 x 65536 40.2 against 37.5, 2048 x 32768 73.9 against 68.2).
+int half_drift_slots_for(const Problem& q, int fv) {
+  if (q.is_bwd && q.numseq > q.at(kT_drift_bwd_max_rows)) return 0;
+  for (int s : {2, 1}) {
+    if (s == 1 && (q.is_bwd || q.numseq > 2)) continue;
+    const int64_t tile = int64_t(8) * s * 64 * fv;
+    if (q.seqlen % tile != 0) continue;
+    const int64_t tiles_per_row = q.seqlen / tile;
+    if (!q.is_bwd && q.numseq >= q.at(128) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
+    const int64_t team = drift_team_size(q, tiles_per_row, s == 2 ? 16 : 8, q.cus);
+    if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
+    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
+    // the teams have to fill at least half the chip, and every member gets a few tiles
+    if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < (q.is_bwd || q.numseq <= 2 ? 2 : 4) * q.cus) continue;
+    return s;
+  }
+  return 0;
+}
 // Returns the tile to use as slots per lane of 8 waves (4: 8192 fp32 elements, 2: 4096), 0 for "not a drift
 // case"; which kernel serves the tile (8 waves, or 16 with half the slots) is the launch planner's business.
 int drift_slots_for(const Problem& q, int fv) {
-  // 16-bit storage: one kernel, forward, tiles of 4096 elements (more per lane do not fit the registers, nor
-  // does any backward).  A step of so little data costs more than the exchange it hides wherever other
-  // kernels fill the chip (bf16 512 x 65536 53 against 37 us, 16 x 1048576 33 against 25 us); one or two very
-  // long rows are what it is for, which no other kernel spreads over every compute unit without waiting
-  // (1 x 33554432 62 against 86 us for look-back tiles, 2 x 16777216 62 against 85 us, 1 x 4194304 14.6
-  // against 16.1 us).
   const bool half = q.dtype != LINREC_DTYPE_F32;
-  if (half && (q.is_bwd || q.numseq > 2)) return 0;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
+  if (half) return half_drift_slots_for(q, fv);
   // More than 2048 rows: the forward only, in tiles of 4096 elements (16 waves of one slot).  Forward / backward in
   // us against one workgroup per row forward and the sweep kernels backward: 4096 x 32768 261.7 / 453.2 against
   // 279.8 / 470.4, 8192 x 32768 543.5 / 965.4 against 565.3 / 964.1, 3000 x 65536 389.9 / 672.2 against 395.8 / 659.5,
@@ -741,6 +764,13 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     int waves = tune && tune->waves > 0 ? tune->waves : 8;
     const int auto_slots = tune && tune->family != LINREC_FAMILY_AUTO ? 0 : drift ? drift_slots_for(q, fv) : sweep_slots_for(q, fv);
     int slots = tune && tune->slots > 0 ? tune->slots : auto_slots > 0 ? auto_slots : (half ? (drift ? 1 : 2) : 4);
+    // 16-bit drift tiles of 8192 elements: 16 waves with one slot each (also what a caller who names the family and
+    // nothing else gets, where the rows are whole tiles of that size)
+    if (drift && half && !(tune && (tune->waves > 0 || tune->slots > 0)) &&
+        (auto_slots == 2 || (auto_slots == 0 && q.seqlen % (int64_t(16) * 64 * fv) == 0))) {
+      waves = 16;
+      slots = 1;
+    }
     // fp32 drift tiles of 4096 elements (every backward, and the forward of rows that are not whole tiles of
     // 8192): 16 waves with one slot each rather than 8 waves with two.  Forward / backward in us: 512 x 65536
     // backward 116.2 against 117.4, 300 x 65536 70.7 against 71.5, 1024 x 65536 229.2 against 231.2, 16 x 1048576

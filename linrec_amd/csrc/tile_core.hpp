@@ -176,6 +176,68 @@ __device__ __forceinline__ void tile_load(TileData<S, VEC, MODE>& d, const RowPt
   }
 }
 
+// A wave's share of one interior tile as it arrives from memory, still in the storage type.  A kernel that keeps
+// loads in flight across the steps of a software pipeline holds 16-bit data this way (half the registers of
+// TileData, and nothing that would have to wait for the loads before the step that uses them).
+template <typename T, int S, int VEC, int MODE>
+struct TilePacked {
+  using V = typename Pack<T, VEC>::type;
+  V xs[S], cs[S], ys[MODE == MODE_BWD ? S : 1];
+  T y_edge;
+};
+
+// The loads of tile_load<..., INTERIOR = true>, in the same order, without the conversion.
+template <int S, int VEC, int MODE, bool DESC, typename T>
+__device__ __forceinline__ void tile_load_packed(TilePacked<T, S, VEC, MODE>& d, const RowPtrs<T>& q, const RowView& rv,
+                                                 int u_wave, int lane) {
+  static_assert(VEC > 1, "whole slots");
+  using V = typename Pack<T, VEC>::type;
+  const long long s_low = DESC ? (long long)rv.nslots - u_wave - S * 64 : (long long)u_wave;
+  const V* bx = reinterpret_cast<const V*>(q.in0) + s_low;
+  const V* bc = reinterpret_cast<const V*>(q.coef) + s_low;
+  const V* by = MODE == MODE_BWD ? reinterpret_cast<const V*>(q.aux) + s_low : nullptr;
+  const unsigned lane_idx = DESC ? 63u - unsigned(lane) : unsigned(lane);
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    d.xs[j] = stream_load(bx + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    d.cs[j] = stream_load(bc + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if constexpr (MODE == MODE_BWD) {
+#pragma unroll
+    for (int j = 0; j < S; ++j) {
+      d.ys[j] = stream_load(by + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    d.y_edge = T(0.0f);
+    if (lane == 63) {
+      const int u_next = u_wave + S * 64;
+      if (u_next < rv.nslots) {
+        const int v = vindex<VEC, DESC>(slot_of<VEC, DESC>(u_next, rv), 0);
+        if (v >= rv.lo && v < rv.hi) d.y_edge = q.aux[v];
+      }
+    }
+  }
+}
+
+template <int S, int VEC, int MODE, bool DESC, typename T>
+__device__ __forceinline__ void tile_unpack(const TilePacked<T, S, VEC, MODE>& k, TileData<S, VEC, MODE>& d) {
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      d.xs[j][i] = float(k.xs[j][DESC ? VEC - 1 - i : i]);
+      d.cs[j][i] = float(k.cs[j][DESC ? VEC - 1 - i : i]);
+      if constexpr (MODE == MODE_BWD) d.ys[j][i] = float(k.ys[j][DESC ? VEC - 1 - i : i]);
+    }
+  }
+  d.y_edge = MODE == MODE_BWD ? float(k.y_edge) : 0.0f;
+}
+
 // Result of the lane- and wave-level scan of a wave's share.
 template <int S, int VEC>
 struct TileScan {
@@ -355,6 +417,55 @@ __device__ __forceinline__ float recompute_entry(const RowPtrs<T> q, const RowVi
     has = true;
   }
   return carry;
+}
+
+// tile_apply_store for an interior tile of 16-bit storage whose saved outputs are still packed: the results are
+// rounded and packed as they are computed, so the batch of stores holds S registers' worth per output tensor and
+// not S * VEC floats.  The caller has folded each slot's map from the wave's entry value into the elements' maps
+// (ex_a = 1, ex_b = 0, and pa[j][0] is a factor like the others, also in the backward).  `y_edge`: the saved output
+// after the wave's last (what lane 63 needs; wave-uniform).
+template <int S, int VEC, int MODE, bool DESC, typename T>
+__device__ __forceinline__ void tile_apply_store_packed(const typename Pack<T, VEC>::type* ys, float y_edge,
+                                                        const TileScan<S, VEC>& r, const RowPtrs<T>& q, const RowView& rv,
+                                                        int u_wave, int lane, bool has_entry, float entry) {
+  using V = typename Pack<T, VEC>::type;
+  const long long s_low = DESC ? (long long)rv.nslots - u_wave - S * 64 : (long long)u_wave;
+  V* b0 = reinterpret_cast<V*>(q.out0) + s_low;
+  V* b1 = MODE == MODE_BWD ? reinterpret_cast<V*>(q.out1) + s_low : nullptr;
+  const unsigned lane_idx = DESC ? 63u - unsigned(lane) : unsigned(lane);
+  V o0[S], o1[MODE == MODE_BWD ? S : 1];
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    const float P = has_entry ? fmaf(entry, r.ex_a[j], r.ex_b[j]) : r.ex_b[j];
+    float r0[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r0[i] = fmaf(r.pa[j][i], P, r.pb[j][i]);  // (the caller has folded the slot's map into pa, pb: also into pa[0])
+    if constexpr (MODE == MODE_BWD) {
+      // d_coeffs needs the saved output one step further along the scan (see tile_apply_store)
+      const float first_of_next = (j + 1 < S) ? read_lane(float(ys[(j + 1) % S][DESC ? VEC - 1 : 0]), 0) : y_edge;
+      const float y_next_slot = shift_down_one_lane(float(ys[j][DESC ? VEC - 1 : 0]), first_of_next);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float y_next = i + 1 < VEC ? float(ys[j][DESC ? VEC - 2 - i : i + 1]) : y_next_slot;
+        o1[j][DESC ? VEC - 1 - i : i] = T(r0[i] * y_next);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o0[j][DESC ? VEC - 1 - i : i] = T(r0[i]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    stream_store(o0[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  if constexpr (MODE == MODE_BWD) {
+#pragma unroll
+    for (int j = 0; j < S; ++j) {
+      stream_store(o1[j], b1 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
 }
 
 // The maps of the NW <= 16 waves of a workgroup lie in LDS.  Every wave folds them for itself by a

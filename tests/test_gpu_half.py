@@ -87,7 +87,14 @@ def _tunings(nat, L):
     if L % 8192 == 0:  # rows of whole tiles: teams that go on from row to row
         out.append(nat.Tuning(nat.FAMILY_SWEEP, 8, 2))
         out.append(nat.Tuning(nat.FAMILY_SWEEP, 8, 2, 2, 1))
-    if L % 4096 == 0:  # the same with tiles stored two steps late (compiled for the forward only)
+    if L % 8192 == 0:  # the same with tiles stored two steps late: 16 waves of one slot, both passes
+        k = L // 8192
+        out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1))                     # team = tiles of a row
+        out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1, 3, 0))               # three teams share the rows
+        out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1, 1, 1))               # one walker takes whole rows
+        if k % 2 == 0:
+            out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1, 2, k // 2))      # two tiles of a row per walker
+    if L % 4096 == 0:  # tiles of 4096 elements in 8 waves (compiled for the forward only)
         k = L // 4096
         out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1), False))            # team = tiles of a row
         out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1, 3, 0), False))      # three teams share the rows
@@ -183,21 +190,28 @@ def test_config_shapes_through_autograd(name, shape, coeffs, reverse, transposed
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
 @pytest.mark.parametrize("reverse", [False, True])
 def test_a_few_very_long_rows(nat, reverse, dtype):
-    """One or two very long rows run forward in teams that fill the launch (four and two collecting waves),
-    three to five rows in teams of up to 64; the backward stays with look-back tiles.  Also with a poll limit
-    of one: every wait of the team members for each other's maps may run out, and the results are the same."""
+    """One or two very long rows run in teams that fill the launch (four and two collecting waves), both passes where
+    the rows are whole tiles of 8192 elements and the forward alone where they are whole tiles of 4096 only; three to
+    five rows with less than four tiles for every compute unit, or ragged ones, run forward in teams of up to 64 and
+    backward in look-back tiles.  Also with a poll limit of one: every wait of the team members for each other's maps
+    may run out, and the results are the same."""
     dev = torch.device("cuda:0")
-    for shape, family, team in [((1, 4096 * 1024), nat.FAMILY_DRIFT, 256), ((2, 4096 * 600), nat.FAMILY_DRIFT, 120),
-                                ((3, 4096 * 300), nat.FAMILY_TEAM, 64), ((5, 4096 * 150 + 24), nat.FAMILY_TEAM, 38)]:
+    D, TM, TL = nat.FAMILY_DRIFT, nat.FAMILY_TEAM, nat.FAMILY_TILE
+    for shape, fwd, bwd in [((1, 8192 * 512), (D, 16, 256), (D, 16, 256)), ((2, 8192 * 300), (D, 16, 100), (D, 16, 100)),
+                            ((2, 4096 * 605), (D, 8, 121), (TL, 8, 1)), ((3, 8192 * 512), (D, 16, 256), (D, 16, 256)),
+                            ((3, 4096 * 300), (TM, 8, 64), (TL, 8, 1)), ((5, 4096 * 150 + 24), (TM, 8, 38), (TL, 8, 1))]:
         x, c, dy = _inputs(shape, dtype, seed=shape[0], coeffs="near1")
         plan = nat.plan(x.to(dev), reverse)
-        assert (plan["family"], plan["tasks"]) == (family, team), plan
-        assert nat.plan(x.to(dev), reverse, True)["family"] == nat.FAMILY_TILE
+        assert (plan["family"], plan["waves"], plan["tasks"]) == fwd, plan
+        plan = nat.plan(x.to(dev), reverse, True)
+        assert (plan["family"], plan["waves"], plan["tasks"]) == bwd, plan
         _run(nat, x, c, dy, reverse, None, f"{dtype} {shape} rev={reverse}")
     x, c, dy = _inputs((1, 4096 * 1024), dtype, seed=7)
+    y_kept = nat.fwd(x.to(dev), c.to(dev), reverse)
     old = nat.lib().linrec_set_spin_limit(1)
     try:
         y = nat.fwd(x.to(dev), c.to(dev), reverse)
+        dx, dc = nat.bwd(dy.to(dev), c.to(dev), y_kept, reverse)
         torch.cuda.synchronize()
     finally:
         nat.lib().linrec_set_spin_limit(old)
@@ -206,3 +220,6 @@ def test_a_few_very_long_rows(nat, reverse, dtype):
         ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
     f64 = lambda t: t.float().numpy().astype(np.float64)
     _check(y, oracle.fwd(f64(x), f64(c), reverse), dtype, "with a poll limit of one")
+    dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y_kept.cpu()), reverse)
+    _check(dx, dx_t, dtype, "d_inputs with a poll limit of one")
+    _check(dc, dc_t, dtype, "d_coeffs with a poll limit of one")

@@ -308,26 +308,39 @@ class TestPlanner:
         assert fam((T["team_min_rows"], (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
         assert fam((T["team_min_rows"] - 1, (1 << 20) + 4)) == nat.FAMILY_TILE      # fewer: look-back tiles
         assert fam((300, 65536), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
-        assert fam((16, 1 << 20), dtype=torch.bfloat16) == nat.FAMILY_TEAM
-        # 16-bit storage, forward: one or two very long rows in one team of the whole launch (tiles of 4096
-        # elements), teams of 64 from three rows on; the backward of fewer than six rows stays with look-back tiles
+        # 16-bit storage: teams whose tiles are stored two steps late (tiles of 8192 elements in 16 waves of one slot)
+        # serve the backward of up to drift_bwd_max_rows rows of whole tiles and the forward of fewer than 128 rows
+        # (up to 255 rows of 32 tiles and more), where the launch has two (forward: four) tiles for every compute unit
         for dt in (torch.bfloat16, torch.float16):
-            q = nat.plan(torch.empty(1, 1 << 25, dtype=dt))
-            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 8, 1, 256, 256), q
+            for shape, bwd in [((1, 1 << 25), False), ((1, 1 << 25), True), ((1, 1 << 22), False), ((1, 1 << 22), True)]:
+                q = nat.plan(torch.empty(shape, dtype=dt), False, bwd)
+                assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 256, 256), q
+            q = nat.plan(torch.empty(16, 1 << 20, dtype=dt))
+            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 128, 256), q
             assert fam((2, 1 << 22), dtype=dt) == D and fam((1, 1 << 20), dtype=dt) == nat.FAMILY_TILE
-            assert [fam((n, 1 << 22), dtype=dt) for n in (3, 4, 5, 6)] == [nat.FAMILY_TEAM] * 4
-            assert [fam((n, 1 << 22), True, dtype=dt) for n in (1, 2, 3, 5, 6)] == [nat.FAMILY_TILE] * 4 + [nat.FAMILY_TEAM]
+            assert fam((1, 1 << 20), True, dtype=dt) == nat.FAMILY_TILE
+            assert [fam((n, 1 << 22), b, dtype=dt) for n in (3, 4, 5, 6) for b in (False, True)] == [D] * 8
+            assert [fam((n, 65536), True, dtype=dt) for n in (127, 300, 512, T["drift_bwd_max_rows"])] == [D] * 4
+            assert fam((T["drift_bwd_max_rows"] + 1, 65536), True, dtype=dt) == ST
+            assert [fam((n, 65536), dtype=dt) for n in (128, 300, 512)] == [W, ST, ST]
+            assert [fam((n, 262144), dtype=dt) for n in (64, 128, 160, 255, 256)] == [D, D, D, D, ST]
+            assert fam((24, 262144), dtype=dt) == nat.FAMILY_TEAM and fam((24, 262144), True, dtype=dt) == D
+            # one or two rows of whole tiles of 4096 elements only: the forward in 8 waves, the backward in look-back tiles
+            q = nat.plan(torch.empty(2, 4096 * 1001, dtype=dt))
+            assert (q["family"], q["waves"], q["slots"], q["tiles_per_row"]) == (D, 8, 1, 1001), q
+            assert fam((2, 4096 * 1001), True, dtype=dt) == nat.FAMILY_TILE
+            # a caller who names the family and nothing else gets the tiles of 8192 elements where the rows are whole ones
+            q = nat.plan(torch.empty(512, 65536, dtype=dt), tuning=nat.Tuning(D))
+            assert (q["waves"], q["slots"], q["tasks"]) == (16, 1, 8), q
             # many rows of exactly two of the stream kernel's tiles: one workgroup walks the row
             assert [fam((n, 16384), b, dtype=dt) for n in (2048, 4096) for b in (False, True)] == [ST] * 4
             assert fam((1024, 16384), dtype=dt) == nat.FAMILY_TILE and fam((2048, 16000), dtype=dt) == nat.FAMILY_TILE
             # rows beyond one per CU get a launch of their own in the backward only
-            tails = lambda n: [nat.plan(torch.empty(n, 65536, dtype=dt), False, b)["tail_rows"] for b in (False, True)]
+            tails = lambda n: [nat.plan(torch.empty(n, 65536 + 8, dtype=dt), False, b)["tail_rows"] for b in (False, True)]
             assert tails(288) == [0, 32] and tails(352) == [0, 96] and tails(400) == [0, 0]
-        # 16-bit backward: one team per row where teams of 256 / rows workgroups fill the chip
-        hb = lambda n: fam((n, 262144), True, dtype=torch.bfloat16)
-        assert [hb(n) for n in (32, 48, 64, 80, 128)] == [nat.FAMILY_TEAM] * 5
-        assert [hb(n) for n in (96, 100, 160)] == [nat.FAMILY_SWEEP] * 3
-        assert fam((64, 262144), dtype=torch.float16) == nat.FAMILY_SWEEP and fam((64, 262144), True) == D
+        # 16-bit backward with less than two tiles for every compute unit: the teams that wait (from 32 rows on)
+        assert fam((100, 32768), True, dtype=torch.bfloat16) == W and fam((100, 32768), dtype=torch.bfloat16) == W
+        assert fam((64, 262144), True) == D
         pf, pb = nat.plan(torch.empty(300, 65536)), nat.plan(torch.empty(300, 65536), False, True)
         assert (pf["tasks"], pf["grid"]) == (8, 256) and (pb["tasks"], pb["grid"]) == (16, 256)
         p = nat.plan(torch.empty(40, 8192 * 24))                    # 24 tiles: teams of 24, 10 of them
@@ -784,6 +797,8 @@ def test_sixteen_bit_types_plan_and_host_path(dtype):
     p = nat.plan(torch.empty(1000, 4096, dtype=dtype))
     assert p["family"] == nat.FAMILY_TILE and p["waves"] * p["slots"] * 64 * 8 >= 4096 and p["slots"] <= 2
     p = nat.plan(torch.empty(16, 1 << 20, dtype=dtype))
+    assert p["family"] == nat.FAMILY_DRIFT and p["vec"] == 8
+    p = nat.plan(torch.empty(16, (1 << 20) + 8, dtype=dtype))
     assert p["family"] == nat.FAMILY_TEAM
     p = nat.plan(torch.empty(256, 262144, dtype=dtype).t())
     assert p["family"] == nat.FAMILY_COLUMN and p["vec"] == 4
