@@ -95,6 +95,16 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   // type until their step comes (half the registers, and no conversion that would have to wait for the loads in
   // the step that issues them).
   constexpr bool PACKED = !std::is_same_v<T, float>;
+  // ... and the forward keeps a scanned tile as its packed inputs plus each slot's map, and scans the elements a second
+  // time when it stores them: a quarter of the registers of the elements' maps, which is what lets a lane hold two
+  // slots of eight elements (a step then moves as many bytes as the fp32 kernels')
+  constexpr bool REPLAY = PACKED && MODE == MODE_FWD;
+  // With two slots to a lane even the packed inputs of three tiles are more than the registers hold: a scanned tile's
+  // packed inputs wait in LDS (every lane its own 16-byte places: no conflicts, no barrier), which the kernel otherwise
+  // leaves unused: two tiles of 64 KB.
+  constexpr bool PARKED = REPLAY && S >= 2;
+  using Packed16 = typename Pack<T, PACKED ? VEC : 4>::type;
+  __shared__ Packed16 sh_park[PARKED ? 2 * NW * S * 2 * 64 : 1];
   using Loaded = std::conditional_t<PACKED, TilePacked<T, S, VEC, MODE>, TileData<S, VEC, MODE>>;
   // A tile that has been scanned and not stored yet.
   struct Pending {
@@ -104,6 +114,7 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     Affine before;  // the waves in front of this one
     Affine total;   // the whole tile's map
     Item it;
+    int park;       // where its packed inputs wait in LDS (0 or 1)
   };
   Loaded D[3];  // tile n lies in D[n % 3]
   Item DI[3];
@@ -246,7 +257,20 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       has_entry = true;
       entry = q.before.b;
     }
-    if constexpr (PACKED) {
+    if constexpr (PARKED) {
+      Loaded k;
+      const Packed16* from = sh_park + ((q.park * NW + wave) * S * 2) * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < S; ++j) {
+        k.xs[j] = from[(2 * j) * 64];
+        k.cs[j] = from[(2 * j + 1) * 64];
+      }
+      tile_replay_store_packed<S, VEC, DESC>(k, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
+                                             t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+    } else if constexpr (REPLAY) {
+      tile_replay_store_packed<S, VEC, DESC>(q.d, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
+                                             t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+    } else if constexpr (PACKED) {
       tile_apply_store_packed<S, VEC, MODE, DESC>(q.d.ys, q.edge, q.r, ptrs_of(q.it.row), rv,
                                                   t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
     } else {
@@ -270,50 +294,46 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
     if (n >= 2 && (wide || wave == 0)) ask(P[OLD].it, w0, w1);
     __builtin_amdgcn_sched_barrier(0);
     if (prefetch) load_next(D[LD], DI[LD]);
-    TileData<S, VEC, MODE> unpacked;
-    TileData<S, VEC, MODE>& d = [&]() -> TileData<S, VEC, MODE>& {
-      if constexpr (PACKED) {
-        tile_unpack<S, VEC, MODE, DESC>(D[PH], unpacked);
-        return unpacked;
-      } else {
-        return D[PH];
-      }
-    }();
     const Item it = DI[PH];
-    if constexpr (MODE == MODE_FWD) {
-      if (it.t == 0 && wave == 0 && lane == 0) d.cs[0][0] = 0.0f;  // the row's first coefficient takes no part
-    }
     Pending& now = P[PH];
-    tile_scan<S, VEC, MODE>(d, now.r);
-    if constexpr (MODE == MODE_FWD) {
-      // a slot's map from the wave's entry value to the slot's is folded into the elements' maps, which leaves
-      // a pending tile two values per element and nothing per slot (16 waves have 128 registers each); nothing
-      // enters a row's first wave, whose factors are therefore zero and never meet a product that overflowed
-      const bool nothing_enters = it.t == 0 && wave == 0;
-#pragma unroll
-      for (int j = 0; j < S; ++j) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
-          now.r.pa[j][i] = nothing_enters ? 0.0f : now.r.pa[j][i] * now.r.ex_a[j];
+    if constexpr (REPLAY) {
+      tile_scan_packed_fwd<S, VEC, DESC>(D[PH], it.t == 0 && wave == 0 && lane == 0, now.r);
+      if constexpr (!PARKED) now.d = D[PH];
+    } else {
+      TileData<S, VEC, MODE> unpacked;
+      TileData<S, VEC, MODE>& d = [&]() -> TileData<S, VEC, MODE>& {
+        if constexpr (PACKED) {
+          tile_unpack<S, VEC, MODE, DESC>(D[PH], unpacked);
+          return unpacked;
+        } else {
+          return D[PH];
         }
-        now.r.ex_a[j] = 1.0f;
-        now.r.ex_b[j] = 0.0f;
+      }();
+      if constexpr (MODE == MODE_FWD) {
+        if (it.t == 0 && wave == 0 && lane == 0) d.cs[0][0] = 0.0f;  // the row's first coefficient takes no part
       }
-    }
-    if constexpr (MODE == MODE_BWD && PACKED) {
-      // 16-bit storage: the same folding in the backward (whose first factor of a slot is one before it), one
-      // register less for each of the three tiles in the works
-      const bool nothing_enters = it.t == 0 && wave == 0;
+      tile_scan<S, VEC, MODE>(d, now.r);
+      if constexpr (MODE == MODE_FWD || PACKED) {
+        // a slot's map from the wave's entry value to the slot's is folded into the elements' maps, which leaves
+        // a pending tile two values per element and nothing per slot (16 waves have 128 registers each); nothing
+        // enters a row's first wave, whose factors are therefore zero and never meet a product that overflowed
+        // (the backward, whose first factor of a slot is one before the folding, only for 16-bit storage, where it
+        // saves a register for each of the three tiles in the works)
+        const bool nothing_enters = it.t == 0 && wave == 0;
 #pragma unroll
-      for (int j = 0; j < S; ++j) {
+        for (int j = 0; j < S; ++j) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
-          now.r.pa[j][i] = nothing_enters ? 0.0f : now.r.pa[j][i] * now.r.ex_a[j];
+          for (int i = 0; i < VEC; ++i) {
+            now.r.pb[j][i] = fmaf(now.r.pa[j][i], now.r.ex_b[j], now.r.pb[j][i]);
+            now.r.pa[j][i] = nothing_enters ? 0.0f : now.r.pa[j][i] * now.r.ex_a[j];
+          }
+          now.r.ex_a[j] = 1.0f;
+          now.r.ex_b[j] = 0.0f;
         }
-        now.r.ex_a[j] = 1.0f;
-        now.r.ex_b[j] = 0.0f;
+      }
+      if constexpr (MODE == MODE_BWD) {
+        now.d = D[PH];
+        if constexpr (PACKED) now.edge = read_lane(d.y_edge, 63);  // (only lane 63 holds it, only lane 63 uses it)
       }
     }
     const int par = n & 1;
@@ -335,9 +355,15 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       const float tile_in = combine(P[OLD], par, n);
       store_pending(P[OLD], tile_in);
     }
-    if constexpr (MODE == MODE_BWD) {
-      now.d = D[PH];
-      if constexpr (PACKED) now.edge = read_lane(d.y_edge, 63);  // (only lane 63 holds it, only lane 63 uses it)
+    if constexpr (PARKED) {
+      // (into the place the tile just stored has left)
+      now.park = n & 1;
+      Packed16* to = sh_park + ((now.park * NW + wave) * S * 2) * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < S; ++j) {
+        to[(2 * j) * 64] = D[PH].xs[j];
+        to[(2 * j + 1) * 64] = D[PH].cs[j];
+      }
     }
     now.it = it;
   };

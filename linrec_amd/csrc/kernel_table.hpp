@@ -69,7 +69,7 @@ KernelGroup kernels_bf16_cols();
 #define DRIFT_TILES_AHEAD(NW, S, VEC, MODE) ((NW) == 16 && (S) == 1 && (VEC) == 4 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
-   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, VEC, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2)>, DT, LINREC_FAMILY_DRIFT, \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, VEC, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2 && (VEC) == 4)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
@@ -168,7 +168,7 @@ KernelGroup kernels_bf16_cols();
   TILE_(TY, 8, 2, 8, 0), TILE_(TY, 16, 2, 8, 0), TILE_(TY, 4, 2, 8, 1), TILE_(TY, 8, 4, 8, 1),  \
   TILE_(TY, 4, 4, 1, 0), TILE_(TY, 4, 4, 1, 1), STREAM_(TY, 8, 2, 8), TEAM_(TY, 8, 2, 8),       \
   TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8),                            \
-  DRIFT_FWD_(TY, 16, 1, 8), DRIFT_BWD_(TY, 16, 1, 8)
+  DRIFT_FWD_(TY, 16, 1, 8), DRIFT_BWD_(TY, 16, 1, 8), DRIFT_FWD_(TY, 16, 2, 8)
 #define HALF_COLUMN_KERNELS(TY)                                                                 \
   GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
   COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16), \

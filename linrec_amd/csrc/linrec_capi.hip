@@ -257,11 +257,12 @@ bool little_work_in_many_rows(const Problem& q) {
   return q.dtype == LINREC_DTYPE_F32 && q.numseq * 4 >= q.cus && q.numseq * q.seqlen <= kT_little_work_max_tiles_per_cu * 8192 * q.cus;
 }
 // The largest team a drift kernel of this geometry serves: a lane of a wave per team mate, in every wave - except
-// 16 waves of two slots, compiled for one collecting wave.
-int64_t drift_max_team(int waves, int slots) { return waves == 16 && slots == 2 ? 64 : int64_t(64) * waves; }
+// 16 waves of two slots of four fp32 elements, compiled for one collecting wave.
+int64_t drift_max_team(int waves, int slots, int vec) { return waves == 16 && slots == 2 && vec == 4 ? 64 : int64_t(64) * waves; }
 // 16-bit storage: tiles of 8192 elements in 16 waves (tiles in flight stay in the storage type, so a lane's eight
-// elements of a slot cost what four fp32 elements do), or of 4096 in 8 waves, forward only, for one or two rows that
-// are not whole tiles of 8192.  Returns 2 or 1 accordingly, 0 for "not a drift case".
+// elements of a slot cost what four fp32 elements do); forward only, tiles of 16384 elements in 16 waves (scanned tiles
+// wait in LDS as packed inputs and are scanned again when they are stored), or of 4096 in 8 waves for one or two rows
+// that are not whole tiles of 8192.  Returns 4, 2 or 1 accordingly, 0 for "not a drift case".
 // The backward wins wherever the fp32 one does (bf16, us, against the table's choice before: 512 x 65536 56.9
 // against 63.8 for one workgroup per row, 300 x 65536 36.3 against 44.0, 2048 x 32768 110.7 against 121.4, 1024 x
 // 131072 220.7 against 246.9; 16 x 1048576 31.5 against 41.8 for one team per row, 64 x 524288 57.2 against 70.5;
@@ -271,15 +272,21 @@ int64_t drift_max_team(int waves, int slots) { return waves == 16 && slots == 2 
 // per row, 64 x 524288 40.7 against 45.2, 96 x 262144 30.9 against 32.9, 16 x 1048576 25.2 against 25.5; rows of 32
 // tiles and more up to 255 of them: 128 x 262144 39.2 against 41.1, 160 x 262144 47.9 against 51.4; but 128 x 65536
 // 14.5 against 12.9, 200 x 65536 19.8 against 16.4, 512 x 65536 40.2 against 37.5, 2048 x 32768 73.9 against 68.2).
+// Its tiles of 16384 elements move as much in a step as the fp32 forward's and serve any number of rows of four such
+// tiles and more (against tiles of 8192 / the table's choice before: 16 x 1048576 20.4 against 24.7 / 25.3 us,
+// 1 x 33554432 38.6 against 42.9, 64 x 524288 37.0 against 39.6, 300 x 65536 24.0 against 25.6 / 26.9 for one workgroup
+// per row, 1024 x 131072 136.6 against 145.9 / 141.4, 512 x 65536 36.7 against 38.6 / 37.3; rows of two tiles:
+// 2048 x 32768 70.9 against 67.9).
 int half_drift_slots_for(const Problem& q, int fv) {
   if (q.is_bwd && q.numseq > q.at(kT_drift_bwd_max_rows)) return 0;
-  for (int s : {2, 1}) {
+  for (int s : {4, 2, 1}) {
+    if (s == 4 && q.is_bwd) continue;
     if (s == 1 && (q.is_bwd || q.numseq > 2)) continue;
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
     const int64_t tiles_per_row = q.seqlen / tile;
-    if (!q.is_bwd && q.numseq >= q.at(128) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
-    const int64_t team = drift_team_size(q, tiles_per_row, s == 2 ? 16 : 8, q.cus);
+    if (s != 4 && !q.is_bwd && q.numseq >= q.at(128) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
+    const int64_t team = drift_team_size(q, tiles_per_row, s == 1 ? 8 : 16, q.cus);
     if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
     if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
     // the teams have to fill at least half the chip, and every member gets a few tiles
@@ -771,6 +778,11 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       waves = 16;
       slots = 1;
     }
+    // ... and its forward tiles of 16384 elements: 16 waves with two slots each
+    if (drift && half && auto_slots == 4 && !(tune && (tune->waves > 0 || tune->slots > 0))) {
+      waves = 16;
+      slots = 2;
+    }
     // fp32 drift tiles of 4096 elements (every backward, and the forward of rows that are not whole tiles of
     // 8192): 16 waves with one slot each rather than 8 waves with two.  Forward / backward in us: 512 x 65536
     // backward 116.2 against 117.4, 300 x 65536 70.7 against 71.5, 1024 x 65536 229.2 against 231.2, 16 x 1048576
@@ -802,7 +814,7 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
                              ? tune->tasks
                              : drift ? drift_team_size(q, tiles_per_row, waves, resident)
                                      : sweep_team_size(tiles_per_row, std::min<int64_t>(kSweepMaxTeam, resident));
-    if (team > (drift ? drift_max_team(waves, slots) : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
+    if (team > (drift ? drift_max_team(waves, slots, fv) : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
     int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
     if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;
@@ -1157,7 +1169,7 @@ int launch(const linrec_plan_t& plan, const Problem& q, const void* in0, const v
     }
     a.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     // (a plan made elsewhere, or edited: never a team the kernel was not compiled for)
-    if (plan.family == LINREC_FAMILY_DRIFT && a.tasks > drift_max_team(k.waves, k.slots)) return LINREC_E_INVALID;
+    if (plan.family == LINREC_FAMILY_DRIFT && a.tasks > drift_max_team(k.waves, k.slots, k.vec)) return LINREC_E_INVALID;
 #ifdef LINREC_PHASE_TIMING
     a.timing = g_timing_buffer;
 #endif

@@ -419,6 +419,79 @@ __device__ __forceinline__ float recompute_entry(const RowPtrs<T> q, const RowVi
   return carry;
 }
 
+// Forward, 16-bit storage, for kernels that store a tile some steps after scanning it: the scan of a packed tile
+// that leaves only each slot's map from the wave's entry value (ex_a, ex_b) and the wave's map (total).  The
+// elements are scanned a second time when the tile is stored (tile_replay_store_packed), from the packed inputs,
+// which take a quarter of the registers of the elements' maps (pa, pb) and the same number of operations.
+// `row_first_lane`: this lane's first element is the row's first, whose coefficient takes no part.
+template <int S, int VEC, bool DESC, typename T>
+__device__ __forceinline__ void tile_scan_packed_fwd(const TilePacked<T, S, VEC, MODE_FWD>& k, bool row_first_lane,
+                                                     TileScan<S, VEC>& r) {
+  float agg_a[S], agg_b[S];
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    float a = float(k.cs[j][DESC ? VEC - 1 : 0]);
+    float b = float(k.xs[j][DESC ? VEC - 1 : 0]);
+    if (j == 0 && row_first_lane) a = 0.0f;
+#pragma unroll
+    for (int i = 1; i < VEC; ++i) {
+      const float c = float(k.cs[j][DESC ? VEC - 1 - i : i]);
+      a *= c;
+      b = fmaf(b, c, float(k.xs[j][DESC ? VEC - 1 - i : i]));
+    }
+    agg_a[j] = a;
+    agg_b[j] = b;
+    __builtin_amdgcn_sched_barrier(0);  // (one slot's unpacked elements at a time)
+  }
+  wave_inclusive_scan<S>(agg_a, agg_b);
+  Affine run = {1.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    const Affine lane_ex = {shift_up_one_lane(agg_a[j], 1.0f), shift_up_one_lane(agg_b[j], 0.0f)};
+    const Affine row_total = {read_lane(agg_a[j], 63), read_lane(agg_b[j], 63)};
+    if (j == 0) {
+      r.ex_a[j] = lane_ex.a;
+      r.ex_b[j] = lane_ex.b;
+    } else {
+      const Affine e = compose(run, lane_ex);
+      r.ex_a[j] = e.a;
+      r.ex_b[j] = e.b;
+    }
+    run = j == 0 ? row_total : compose(run, row_total);
+  }
+  r.total = run;
+}
+
+// ... and the second scan: every lane runs the recurrence over its slots' elements from the value that enters the
+// slot, rounds and packs the results as they come, and the stores go out back to back.
+template <int S, int VEC, bool DESC, typename T>
+__device__ __forceinline__ void tile_replay_store_packed(const TilePacked<T, S, VEC, MODE_FWD>& k, const TileScan<S, VEC>& r,
+                                                         bool row_first_lane, const RowPtrs<T>& q, const RowView& rv,
+                                                         int u_wave, int lane, bool has_entry, float entry) {
+  using V = typename Pack<T, VEC>::type;
+  const long long s_low = DESC ? (long long)rv.nslots - u_wave - S * 64 : (long long)u_wave;
+  V* b0 = reinterpret_cast<V*>(q.out0) + s_low;
+  const unsigned lane_idx = DESC ? 63u - unsigned(lane) : unsigned(lane);
+  V o[S];
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    float y = has_entry ? fmaf(entry, r.ex_a[j], r.ex_b[j]) : r.ex_b[j];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float x = float(k.xs[j][DESC ? VEC - 1 - i : i]);
+      const float c = float(k.cs[j][DESC ? VEC - 1 - i : i]);
+      y = (i == 0 && j == 0 && row_first_lane) ? x : fmaf(y, c, x);
+      o[j][DESC ? VEC - 1 - i : i] = T(y);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // (one slot's unpacked elements at a time)
+  }
+#pragma unroll
+  for (int j = 0; j < S; ++j) {
+    stream_store(o[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 // tile_apply_store for an interior tile of 16-bit storage whose saved outputs are still packed: the results are
 // rounded and packed as they are computed, so the batch of stores holds S registers' worth per output tensor and
 // not S * VEC floats.  The caller has folded each slot's map from the wave's entry value into the elements' maps

@@ -94,6 +94,13 @@ def _tunings(nat, L):
         out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1, 1, 1))               # one walker takes whole rows
         if k % 2 == 0:
             out.append(nat.Tuning(nat.FAMILY_DRIFT, 16, 1, 2, k // 2))      # two tiles of a row per walker
+    if L % 16384 == 0:  # forward only: tiles of 16384 elements, which wait in LDS as packed inputs and are scanned twice
+        k = L // 16384
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 16, 2), False))
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 16, 2, 3, 0), False))
+        out.append((nat.Tuning(nat.FAMILY_DRIFT, 16, 2, 1, 1), False))
+        if k % 2 == 0:
+            out.append((nat.Tuning(nat.FAMILY_DRIFT, 16, 2, 2, k // 2), False))
     if L % 4096 == 0:  # tiles of 4096 elements in 8 waves (compiled for the forward only)
         k = L // 4096
         out.append((nat.Tuning(nat.FAMILY_DRIFT, 8, 1), False))            # team = tiles of a row
@@ -197,16 +204,24 @@ def test_a_few_very_long_rows(nat, reverse, dtype):
     may run out, and the results are the same."""
     dev = torch.device("cuda:0")
     D, TM, TL = nat.FAMILY_DRIFT, nat.FAMILY_TEAM, nat.FAMILY_TILE
-    for shape, fwd, bwd in [((1, 8192 * 512), (D, 16, 256), (D, 16, 256)), ((2, 8192 * 300), (D, 16, 100), (D, 16, 100)),
-                            ((2, 4096 * 605), (D, 8, 121), (TL, 8, 1)), ((3, 8192 * 512), (D, 16, 256), (D, 16, 256)),
-                            ((3, 4096 * 300), (TM, 8, 64), (TL, 8, 1)), ((5, 4096 * 150 + 24), (TM, 8, 38), (TL, 8, 1))]:
+    for shape, fwd, bwd in [((1, 8192 * 512), (D, 16, 1, 256), (D, 16, 1, 256)), ((2, 8192 * 300), (D, 16, 1, 100), (D, 16, 1, 100)),
+                            ((2, 4096 * 605), (D, 8, 1, 121), (TL, 8, 4, 1)), ((3, 8192 * 512), (D, 16, 1, 256), (D, 16, 1, 256)),
+                            ((4, 16384 * 512), (D, 16, 2, 256), (D, 16, 1, 256)), ((5, 16384 * 231), (D, 16, 2, 231), (D, 16, 1, 231)),
+                            ((3, 4096 * 300), (TM, 8, 4, 64), (TL, 8, 4, 1)), ((5, 4096 * 150 + 24), (TM, 8, 4, 38), (TL, 8, 4, 1))]:
         x, c, dy = _inputs(shape, dtype, seed=shape[0], coeffs="near1")
         plan = nat.plan(x.to(dev), reverse)
-        assert (plan["family"], plan["waves"], plan["tasks"]) == fwd, plan
+        assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == fwd, plan
         plan = nat.plan(x.to(dev), reverse, True)
-        assert (plan["family"], plan["waves"], plan["tasks"]) == bwd, plan
+        assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == bwd, plan
         _run(nat, x, c, dy, reverse, None, f"{dtype} {shape} rev={reverse}")
-    x, c, dy = _inputs((1, 4096 * 1024), dtype, seed=7)
+    # (the last: forward in tiles of 16384 elements, backward in tiles of 8192)
+    for shape in ((1, 4096 * 1024), (8, 16384 * 128)):
+        _poll_limit_one(nat, shape, dtype, reverse)
+
+
+def _poll_limit_one(nat, shape, dtype, reverse):
+    dev = torch.device("cuda:0")
+    x, c, dy = _inputs(shape, dtype, seed=7)
     y_kept = nat.fwd(x.to(dev), c.to(dev), reverse)
     old = nat.lib().linrec_set_spin_limit(1)
     try:

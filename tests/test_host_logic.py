@@ -307,23 +307,30 @@ class TestPlanner:
         assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
         assert fam((T["team_min_rows"], (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
         assert fam((T["team_min_rows"] - 1, (1 << 20) + 4)) == nat.FAMILY_TILE      # fewer: look-back tiles
-        assert fam((300, 65536), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
-        # 16-bit storage: teams whose tiles are stored two steps late (tiles of 8192 elements in 16 waves of one slot)
-        # serve the backward of up to drift_bwd_max_rows rows of whole tiles and the forward of fewer than 128 rows
-        # (up to 255 rows of 32 tiles and more), where the launch has two (forward: four) tiles for every compute unit
+        assert fam((300, 65536 + 8), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
+        # 16-bit storage: teams whose tiles are stored two steps late serve the backward of up to drift_bwd_max_rows
+        # rows of whole tiles of 8192 elements (16 waves of one slot) and the forward of any number of rows of four and
+        # more tiles of 16384 elements (16 waves of two slots), where the launch has two (forward: four) tiles for every
+        # compute unit; the forward of fewer than 128 rows (up to 255 of 32 tiles and more) also in tiles of 8192
         for dt in (torch.bfloat16, torch.float16):
-            for shape, bwd in [((1, 1 << 25), False), ((1, 1 << 25), True), ((1, 1 << 22), False), ((1, 1 << 22), True)]:
+            for shape, bwd, slots in [((1, 1 << 25), False, 2), ((1, 1 << 25), True, 1), ((1, 1 << 22), False, 1), ((1, 1 << 22), True, 1)]:
                 q = nat.plan(torch.empty(shape, dtype=dt), False, bwd)
-                assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 256, 256), q
+                assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, slots, 256, 256), q
             q = nat.plan(torch.empty(16, 1 << 20, dtype=dt))
-            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 128, 256), q
+            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 2, 64, 256), q
+            q = nat.plan(torch.empty(16, 8192 * 129, dtype=dt))
+            assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 43, 215), q  # (five teams of 43: 215 of 256 workgroups)
             assert fam((2, 1 << 22), dtype=dt) == D and fam((1, 1 << 20), dtype=dt) == nat.FAMILY_TILE
             assert fam((1, 1 << 20), True, dtype=dt) == nat.FAMILY_TILE
             assert [fam((n, 1 << 22), b, dtype=dt) for n in (3, 4, 5, 6) for b in (False, True)] == [D] * 8
             assert [fam((n, 65536), True, dtype=dt) for n in (127, 300, 512, T["drift_bwd_max_rows"])] == [D] * 4
             assert fam((T["drift_bwd_max_rows"] + 1, 65536), True, dtype=dt) == ST
-            assert [fam((n, 65536), dtype=dt) for n in (128, 300, 512)] == [W, ST, ST]
-            assert [fam((n, 262144), dtype=dt) for n in (64, 128, 160, 255, 256)] == [D, D, D, D, ST]
+            assert [fam((n, 65536), dtype=dt) for n in (128, 200, 256, 300, 512, 5000)] == [W, ST, D, D, D, D]
+            assert [fam((n, 32768), dtype=dt) for n in (512, 2048)] == [ST, ST]       # rows of two tiles of 16384
+            assert [fam((n, 8192 * 9), dtype=dt) for n in (120, 128, 300)] == [D, W, ST]
+            assert [fam((n, 8192 * 33), dtype=dt) for n in (64, 128, 160, 250, 256)] == [D, D, D, D, ST]
+            q = nat.plan(torch.empty(512, 65536, dtype=dt))
+            assert (q["waves"], q["slots"], q["tasks"], q["grid"]) == (16, 2, 4, 256), q
             assert fam((24, 262144), dtype=dt) == nat.FAMILY_TEAM and fam((24, 262144), True, dtype=dt) == D
             # one or two rows of whole tiles of 4096 elements only: the forward in 8 waves, the backward in look-back tiles
             q = nat.plan(torch.empty(2, 4096 * 1001, dtype=dt))
@@ -791,7 +798,7 @@ def test_logc_and_dim_options(reverse):
 def test_sixteen_bit_types_plan_and_host_path(dtype):
     """16-bit storage: slots hold eight elements, at most two slots per lane, same families."""
     names = nat.kernel_table()
-    p = nat.plan(torch.empty(512, 65536, dtype=dtype))
+    p = nat.plan(torch.empty(512, 65536 + 8, dtype=dtype))
     assert p["family"] == nat.FAMILY_STREAM and p["vec"] == 8 and p["slots"] == 2
     assert names[p["kernel_id"]].startswith("f16_" if dtype == torch.float16 else "bf16_")
     p = nat.plan(torch.empty(1000, 4096, dtype=dtype))
