@@ -285,12 +285,18 @@ int half_drift_slots_for(const Problem& q, int fv) {
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
     const int64_t tiles_per_row = q.seqlen / tile;
-    if (s != 4 && !q.is_bwd && q.numseq >= q.at(128) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
+    if (s != 4 && !q.is_bwd && q.numseq > q.at(kT_half_drift_fwd_small_tiles_max_rows) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
     const int64_t team = drift_team_size(q, tiles_per_row, s == 1 ? 8 : 16, q.cus);
     if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
     if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
-    // the teams have to fill at least half the chip, and every member gets a few tiles
-    if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < (q.is_bwd || q.numseq <= 2 ? 2 : 4) * q.cus) continue;
+    // the teams have to fill at least half the chip, and every member gets a few tiles: the backward and a few rows'
+    // forward (fewer than a quarter of the compute units) as many for each compute unit as the generated table says
+    // (the forward's in tiles of 16384 elements, so twice as many of 8192), more rows forward four of them (200 x 65536
+    // with three: 17.3 against 16.2 us for one workgroup per row), one or two rows two
+    const int64_t per_cu = q.is_bwd ? kT_half_drift_bwd_min_tiles_per_cu
+                           : q.numseq <= 2 ? (s == 1 ? 4 : 2)
+                                           : (q.numseq * 4 < q.cus ? kT_half_drift_fwd_min_tiles_per_cu : 4) * (s == 4 ? 1 : 2);
+    if (std::min(q.numseq, q.cus / team) * team * 2 < q.cus || q.numseq * tiles_per_row < per_cu * q.cus) continue;
     return s;
   }
   return 0;

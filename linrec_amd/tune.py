@@ -280,9 +280,9 @@ class Crossover:
     kind 'first_high': the threshold is the smallest value from which `high` is faster on all larger values
     tried; 'last_low': the largest value up to which `low` is at least as fast on all smaller values tried."""
 
-    def __init__(self, name, what, values, shape, low, high, passes=("fwd", "bwd"), kind="first_high"):
+    def __init__(self, name, what, values, shape, low, high, passes=("fwd", "bwd"), kind="first_high", dtype=torch.float32):
         self.name, self.what, self.values, self.shape = name, what, values, shape
-        self.low, self.high, self.passes, self.kind = low, high, passes, kind
+        self.low, self.high, self.passes, self.kind, self.dtype = low, high, passes, kind, dtype
 
 
 def _t(family, waves=0, slots=0, carry=-1, tasks=0):
@@ -321,16 +321,31 @@ CROSSOVERS = [
     Crossover("drift_bwd_short_rows_min_rows", "backward of rows of four tiles of 4096 elements: one workgroup per "
               "row against drift teams, by the number of rows", [128, 256, 384, 512, 768, 1024, 2048],
               lambda v: (v, 16384), _both(_t(nat.FAMILY_STREAM)), _DRIFT_SMALL, passes=("bwd",)),
+    # 16-bit storage (measured on bf16; fp16 moves the same bytes)
+    Crossover("half_drift_fwd_small_tiles_max_rows", "bf16 forward of rows that are whole tiles of 8192 elements but not "
+              "of 16384 (nine tiles): drift teams against one workgroup per row, or sweep teams, by the number of rows",
+              [64, 96, 112, 127, 144, 160, 200, 256], lambda v: (v, 8192 * 9), _DRIFT_SMALL,
+              [_both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))], passes=("fwd",), kind="last_low", dtype=torch.bfloat16),
+    Crossover("half_drift_fwd_min_tiles_per_cu", "bf16 forward of 16 long rows: look-back tiles, one team per row or sweep "
+              "teams against drift teams with tiles of 16384 elements, by the tiles per compute unit",
+              [1, 2, 3, 4, 6, 8], lambda v: (16, v * 262144),
+              [_both(_t(nat.FAMILY_TILE)), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))],
+              _both(_t(nat.FAMILY_DRIFT, 16, 2)), passes=("fwd",), dtype=torch.bfloat16),
+    Crossover("half_drift_bwd_min_tiles_per_cu", "bf16 backward of 16 long rows: look-back tiles, one team per row or sweep "
+              "teams against drift teams with tiles of 8192 elements, by the tiles per compute unit",
+              [1, 2, 3, 4, 6, 8], lambda v: (16, v * 131072),
+              [_both(_t(nat.FAMILY_TILE)), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))],
+              _DRIFT_SMALL, passes=("bwd",), dtype=torch.bfloat16),
 ]
 
 
-def _time_tunings(shape, tunings, passes, sets=3, iters=30, warmup=6, device="cuda:0", rounds=2):
+def _time_tunings(shape, tunings, passes, sets=3, iters=30, warmup=6, device="cuda:0", rounds=2, dtype=torch.float32):
     """Microseconds of the listed passes added up, for each {pass: Tuning} of `tunings` on tensors of `shape`
     (the candidates take turns, the least of `rounds` counts); inf where the library has no such kernel."""
     dev = torch.device(device)
     bufs = []
     for _ in range(sets):
-        x, c, dy = (f(shape, device=dev) for f in (torch.randn, torch.rand, torch.randn))
+        x, c, dy = (f(shape, device=dev).to(dtype) for f in (torch.randn, torch.rand, torch.randn))
         y = nat.fwd(x, c)
         bufs.append((x, c, dy, y, torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)))
     best = [float("inf")] * len(tunings)
@@ -354,13 +369,20 @@ def _time_tunings(shape, tunings, passes, sets=3, iters=30, warmup=6, device="cu
     return best
 
 
-def measure_crossover(x, log=None):
-    """(threshold, [(value, shape, us_low, us_high)]) of one Crossover on the current device."""
+STICKY = 0.03  # a threshold only moves past values where one side is more than this fraction faster
+
+
+def measure_crossover(x, log=None, current=None):
+    """(threshold, [(value, shape, us_low, us_high)]) of one Crossover on the current device.
+    `current`: the value in force.  Where two kernels' curves cross at a shallow angle the crossing moves with the box
+    and the run; the value in force is kept unless some value tried between it and the newly measured crossing
+    shows one side more than STICKY faster (either choice costs less than that in between)."""
     rows = []
     for v in x.values:
         lows = x.low if isinstance(x.low, list) else [x.low]
-        times = _time_tunings(x.shape(v), lows + [x.high], x.passes)
-        lo, hi = min(times[:-1]), times[-1]
+        highs = x.high if isinstance(x.high, list) else [x.high]
+        times = _time_tunings(x.shape(v), lows + highs, x.passes, dtype=x.dtype)
+        lo, hi = min(times[:len(lows)]), min(times[len(lows):])
         rows.append((v, x.shape(v), lo, hi))
         if log:
             log(f"{x.name}: {v} {x.shape(v)} low {lo:.1f} us high {hi:.1f} us")
@@ -377,16 +399,28 @@ def measure_crossover(x, log=None):
             k += 1
         # (never at least as fast: one below the smallest value tried)
         threshold = rows[k - 1][0] if k > 0 else rows[0][0] - 1
+    if current is not None and current != threshold:
+        # values whose choice differs between the two thresholds
+        if x.kind == "first_high":
+            between = [(lo, hi) for v, _, lo, hi in rows if min(current, threshold) <= v < max(current, threshold)]
+        else:
+            between = [(lo, hi) for v, _, lo, hi in rows if min(current, threshold) < v <= max(current, threshold)]
+        if all(abs(lo - hi) <= STICKY * min(lo, hi) for lo, hi in between):
+            if log:
+                log(f"{x.name}: measured {threshold}, within {STICKY:.0%} of the value in force everywhere in between: {current} kept")
+            threshold = current
     return threshold, rows
 
 
-TABLE_HEADER = """// Crossover thresholds of the launch planner for long rows on the unit-stride axis (fp32), on the full part (256
-// compute units; the planner scales row counts to the device in hand).
+TABLE_HEADER = """// Crossover thresholds of the launch planner for long rows on the unit-stride axis (fp32; the half_* ones for 16-bit
+// storage), on the full part (256 compute units; the planner scales row counts to the device in hand).
 //
 // GENERATED by `python -m linrec_amd.tune --write-table` (the counterpart of the table the reference's grid search
 // writes, eval/tune.py:104-134): every line is the smallest value of the swept quantity from which the second
 // kernel was faster than the first on all larger values tried (or the largest up to which the first held its own);
-// the timings behind each line stand above it.  Edit by re-running the command on the device, not by hand.
+// the timings behind each line stand above it.  A value in force is kept where every value tried between it and the
+// new crossing has the two kernels within 3 % of each other (shallow crossings move with the box and the run).
+// Edit by re-running the command on the device, not by hand.
 //
 // LINREC_THRESHOLD(name, value)
 """
@@ -405,7 +439,7 @@ def write_table(path=None, only=None, log=None):
             out.append("// (not measured in this run: value kept)")
             out.append(f"LINREC_THRESHOLD({x.name}, {current[x.name]})")
             continue
-        threshold, rows = measure_crossover(x, log)
+        threshold, rows = measure_crossover(x, log, current.get(x.name))
         passes = " + ".join(x.passes)
         for v, shape, lo, hi in rows:
             out.append(f"//   {v:>6}  {shape[0]} x {shape[1]}: {passes} {lo:.1f} us against {hi:.1f} us")

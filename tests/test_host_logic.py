@@ -327,11 +327,20 @@ class TestPlanner:
             assert fam((T["drift_bwd_max_rows"] + 1, 65536), True, dtype=dt) == ST
             assert [fam((n, 65536), dtype=dt) for n in (128, 200, 256, 300, 512, 5000)] == [W, ST, D, D, D, D]
             assert [fam((n, 32768), dtype=dt) for n in (512, 2048)] == [ST, ST]       # rows of two tiles of 16384
-            assert [fam((n, 8192 * 9), dtype=dt) for n in (120, 128, 300)] == [D, W, ST]
+            # rows of whole tiles of 8192 elements only: up to half_drift_fwd_small_tiles_max_rows rows, and up to 255
+            # rows of 32 tiles and more
+            few = T["half_drift_fwd_small_tiles_max_rows"]
+            assert fam((few, 8192 * 41), dtype=dt) == D and fam((few + 1, 8192 * 31), dtype=dt) != D
+            assert [fam((n, 8192 * 9), dtype=dt) for n in (128, 300)] == [W, ST]
             assert [fam((n, 8192 * 33), dtype=dt) for n in (64, 128, 160, 250, 256)] == [D, D, D, D, ST]
+            # a few rows: the tiles per compute unit the table asks for (forward: of 16384 elements)
+            for bwd, per_cu, tile in ((False, T["half_drift_fwd_min_tiles_per_cu"], 16384), (True, T["half_drift_bwd_min_tiles_per_cu"], 8192)):
+                assert fam((16, per_cu * 16 * tile), bwd, dtype=dt) == D
+                assert fam((16, (per_cu * 16 - 1) * tile), bwd, dtype=dt) != D or (not bwd and per_cu * 16 - 1 >= 64)
             q = nat.plan(torch.empty(512, 65536, dtype=dt))
             assert (q["waves"], q["slots"], q["tasks"], q["grid"]) == (16, 2, 4, 256), q
-            assert fam((24, 262144), dtype=dt) == nat.FAMILY_TEAM and fam((24, 262144), True, dtype=dt) == D
+            assert fam((24, 262144), dtype=dt) == nat.FAMILY_TEAM
+            assert fam((24, 262144), True, dtype=dt) == (D if 24 * 32 >= 256 * T["half_drift_bwd_min_tiles_per_cu"] else nat.FAMILY_TEAM)
             # one or two rows of whole tiles of 4096 elements only: the forward in 8 waves, the backward in look-back tiles
             q = nat.plan(torch.empty(2, 4096 * 1001, dtype=dt))
             assert (q["family"], q["waves"], q["slots"], q["tiles_per_row"]) == (D, 8, 1, 1001), q
