@@ -244,7 +244,7 @@ def launch_model(shape, sets=3, iters=40, warmup=8, device="cuda:0"):
             t = _event_ms(lambda i: nat.fwd(srcs[i % sets][0], srcs[i % sets][1], False, out=dsts[i % sets][0]), iters, warmup)
 
         def row(label, ms, ends=None):
-            r = {"pass": what, "launch": label, "us": ms * 1e3, "GBps": bpe * n / ms / 1e6, "of_8_TBps": bpe * n / ms / 1e6 / 8000}
+            r = {"pass": what, "launch": label, "us": ms * 1e3, "GBps": bpe * n / ms / 1e6, "pct_of_8_TBps": round(bpe * n / ms / 1e6 / 80, 1)}
             r.update({"first_end_us": float("nan"), "mean_end_us": float("nan"), "last_end_us": float("nan")} if ends is None else ends)
             rows.append(r)
 
