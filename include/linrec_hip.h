@@ -66,12 +66,14 @@ extern "C" {
                                   a wave takes (4 or 2) */
 
 #define LINREC_FAMILY_DRIFT 10  /* the SWEEP launch shape with the exchange between team mates off the critical
-                                  path: a scanned tile is kept in registers and stored two steps late, by which
-                                  time the value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
+                                  path: a scanned tile is kept (in registers; the 16-bit forward's tiles of two
+                                  slots as packed inputs in LDS) and stored two steps late, by which time the
+                                  value entering it has arrived without anybody waiting.  Tuning as SWEEP, with
                                   teams of up to 64 a wave: beyond 64 every wave collects maps.  Compiled (waves x slots):
                                   fp32 forward 8 x 4, 8 x 2, 4 x 4, 16 x 1 and 16 x 2 (the last for teams of at most
-                                  64 only), fp32 backward 8 x 2 and 16 x 1; 16-bit storage 8 x 1, forward only.
-                                  The planner's picks are the 16-wave ones, and 8 x 4 forward for teams beyond 64 */
+                                  64 only), fp32 backward 8 x 2 and 16 x 1; 16-bit storage (slots of eight
+                                  elements) forward 16 x 2, 16 x 1 and 8 x 1, backward 16 x 1.
+                                  The planner's picks are the 16-wave ones, and 8 x 4 forward for fp32 teams beyond 64 */
 
 #define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
                                    of workgroups share a block of rows and take its steps along the scan axis in
