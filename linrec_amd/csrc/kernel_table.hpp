@@ -65,7 +65,8 @@ KernelGroup kernels_bf16_cols();
 // tile ahead in 16 waves had beaten by 1 to 4 %: 512 x 65536 112.4 against 117.5, 300 x 65536 68.3 against 71.2,
 // 16 x 1048576 60.1 against 63.6, 1 x 33554432 111.6 against 124.5); the forward gains nothing from it.
 // (16-bit storage, eight elements per slot: a second tile does not fit the backward's registers and brings the
-// forward nothing: bf16 512 x 65536 40.2 against 40.4 us, 16 x 1048576 25.2 against 25.0)
+// forward nothing: one slot bf16 512 x 65536 40.2 against 40.4 us, 16 x 1048576 25.2 against 25.0; two slots
+// 512 x 65536 37.1 against 36.7, 16 x 1048576 23.3 against 20.4, 300 x 65536 22.8 against 24.0)
 #define DRIFT_TILES_AHEAD(NW, S, VEC, MODE) ((NW) == 16 && (S) == 1 && (VEC) == 4 && linrec::MODE == linrec::MODE_BWD ? 2 : 1)
 #define DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                        \
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
