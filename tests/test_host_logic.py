@@ -44,6 +44,29 @@ def test_planner_thresholds_come_from_the_generated_table():
         assert block.count(" us against ") == len(x.values), x.name
 
 
+def test_table_writer_keeps_a_value_in_force_across_a_shallow_crossing(monkeypatch):
+    """The threshold writer on timings given by hand: the crossing is found from the measured curves, and a value in
+    force is kept unless some value between it and the new crossing shows one kernel more than 3 % faster."""
+    from linrec_amd import tune
+    curves = {}
+    monkeypatch.setattr(tune, "_time_tunings", lambda shape, tunings, passes, **kw: list(curves[shape[0]]))
+    mk = lambda kind: tune.Crossover("t", "test", [2, 4, 6, 8], lambda v: (v, 1024), {"fwd": None}, {"fwd": None},
+                                     passes=("fwd",), kind=kind)
+    # (low, high) per value: high takes over from 6 on, 2 % ahead at 4
+    curves.update({2: (10.0, 11.0), 4: (20.0, 19.6), 6: (30.0, 25.0), 8: (40.0, 33.0)})
+    assert tune.measure_crossover(mk("first_high"))[0] == 4          # smallest value from which high wins
+    assert tune.measure_crossover(mk("last_low"))[0] == 2            # largest value up to which low holds
+    assert tune.measure_crossover(mk("first_high"), current=6)[0] == 6   # 4 is within 3 %: the value in force stays
+    assert tune.measure_crossover(mk("first_high"), current=8)[0] == 4   # 6 is 17 % apart: it moves
+    assert tune.measure_crossover(mk("last_low"), current=4)[0] == 4     # (last_low 4 means: low up to 4; 4 is within 3 %)
+    assert tune.measure_crossover(mk("last_low"), current=6)[0] == 2     # low at 6 costs 20 %
+    # never faster / always faster: one past the ends
+    curves.update({v: (1.0, 2.0) for v in (2, 4, 6, 8)})
+    assert tune.measure_crossover(mk("first_high"))[0] == 9 and tune.measure_crossover(mk("last_low"))[0] == 8
+    curves.update({v: (2.0, 1.0) for v in (2, 4, 6, 8)})
+    assert tune.measure_crossover(mk("first_high"))[0] == 2 and tune.measure_crossover(mk("last_low"))[0] == 1
+
+
 def test_error_strings():
     lib = nat.lib()
     for code in (0, -1, -2, -3, -4, -5):
