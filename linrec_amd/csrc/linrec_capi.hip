@@ -307,12 +307,9 @@ int drift_slots_for(const Problem& q, int fv) {
   const bool half = q.dtype != LINREC_DTYPE_F32;
   if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.elem_stride != 1) return 0;
   if (half) return half_drift_slots_for(q, fv);
-  // More than 2048 rows: the forward only, in tiles of 4096 elements (16 waves of one slot).  Forward / backward in
-  // us against one workgroup per row forward and the sweep kernels backward: 4096 x 32768 261.7 / 453.2 against
-  // 279.8 / 470.4, 8192 x 32768 543.5 / 965.4 against 565.3 / 964.1, 3000 x 65536 389.9 / 672.2 against 395.8 / 659.5,
-  // 4096 x 65536 532.2 / 948.0 against 543.9 / 934.5 (tiles of 8192 in 16 waves of two slots: 271.0, 569.5, 391.9,
-  // 540.6 forward).
-  const bool many_rows = q.numseq > q.at(2048);
+  // More than 2048 rows: the forward gains as well (us, against one workgroup per row: 4096 x 32768 266.0 against
+  // 274.3, 4096 x 40960 335.3 against 360.1, 4096 x 16384 128.9 against 138.8), in the same tiles of 8192 elements as
+  // fewer rows (tiles of 4096: 269.2, 340.2, 139.3).
   if (q.is_bwd && q.numseq > q.at(kT_drift_bwd_max_rows)) return 0;
   // The backward of 16 to 127 rows with little work in all stays with the sweep kernels' tiles of 16384 elements
   // (24 x 262144 25.3 against 26.3 us, 40 x 196608 27.0 against 30.8 us; but 100 x 131072 55.1 against 48.5 us,
@@ -326,12 +323,16 @@ int drift_slots_for(const Problem& q, int fv) {
   for (int s : {4, 2, 1}) {
     if (half != (s == 1)) continue;
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
-    if (many_rows && s == 4) continue;
     const int64_t tile = int64_t(8) * s * 64 * fv;
     if (q.seqlen % tile != 0) continue;
     const int64_t tiles_per_row = q.seqlen / tile;
     const int64_t team = drift_team_size(q, tiles_per_row, 8, q.cus);
-    if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
+    // the forward's tiles of 8192 elements: as many tiles a row as the generated table says, and from its number of
+    // rows on also rows of two tiles in teams of two (us, against one workgroup per row: 2048 x 16384 66.2 against 69.3,
+    // 4096 x 16384 128.9 against 138.8; but 600 x 16384 22.6 against 22.1, 1024 x 16384 34.5 against 35.0)
+    const int64_t least_tiles = s != 4 ? kSweepMinTiles
+                                : q.numseq >= q.at(kT_drift_fwd_two_tiles_min_rows) ? 2 : kT_drift_fwd_min_tiles_per_row;
+    if (tiles_per_row < least_tiles || team < least_tiles) continue;
     // (a caller that can only give so much workspace is served by the kernels that need less)
     if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
     // fp32 rows of fewer than eight tiles of 4096 elements: one workgroup per row does as well or better

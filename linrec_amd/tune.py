@@ -321,6 +321,14 @@ CROSSOVERS = [
     Crossover("drift_bwd_short_rows_min_rows", "backward of rows of four tiles of 4096 elements: one workgroup per "
               "row against drift teams, by the number of rows", [128, 256, 384, 512, 768, 1024, 2048],
               lambda v: (v, 16384), _both(_t(nat.FAMILY_STREAM)), _DRIFT_SMALL, passes=("bwd",)),
+    Crossover("drift_fwd_min_tiles_per_row", "forward of 600 rows of whole tiles of 8192 elements: one workgroup per "
+              "row, or sweep teams, against drift teams, by the tiles of a row", [2, 3, 4, 5, 6],
+              lambda v: (600, v * 8192), [_both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_SWEEP, 8, 4))], _DRIFT,
+              passes=("fwd",)),
+    Crossover("drift_fwd_two_tiles_min_rows", "forward of rows of two tiles of 8192 elements: one workgroup per row, or "
+              "sweep teams, against drift teams of two, by the number of rows", [512, 768, 1024, 1536, 2048, 3072, 4096],
+              lambda v: (v, 16384), [_both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))], _DRIFT,
+              passes=("fwd",)),
     # 16-bit storage (measured on bf16; fp16 moves the same bytes)
     Crossover("half_drift_fwd_small_tiles_max_rows", "bf16 forward of rows that are whole tiles of 8192 elements but not "
               "of 16384 (nine tiles): drift teams against one workgroup per row, or sweep teams, by the number of rows",

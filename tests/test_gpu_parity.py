@@ -660,18 +660,21 @@ def test_little_work_in_many_rows_goes_to_small_teams_with_the_largest_tiles(nat
 
 @pytest.mark.parametrize("reverse", [False, True])
 def test_more_than_2048_rows_of_whole_tiles_run_forward_in_teams(nat, reverse):
-    """Beyond 2048 rows the forward still goes to the teams whose tiles are stored two steps late (tiles of 4096
-    elements, 16 waves) where a row has enough such tiles (the planner's generated threshold), the backward to them
-    as well up to its own threshold, else to the teams that wait or to one workgroup per row."""
+    """Beyond 2048 rows the forward still goes to the teams whose tiles are stored two steps late: tiles of 8192
+    elements in 16 waves of two slots (rows of two such tiles included), tiles of 4096 in 16 waves of one slot where
+    only those divide the row and it has enough of them (the planner's generated thresholds); the backward to them as
+    well up to its own threshold, else to the teams that wait or to one workgroup per row."""
     dev = torch.device("cuda:0")
-    k = nat.plan_thresholds()["drift_min_small_tiles_per_row"]
+    T = nat.plan_thresholds()
+    k = T["drift_min_small_tiles_per_row"]
     k += 1 - k % 2  # (odd: whole tiles of 4096 elements but not of 8192)
-    for n, L, team in [(2100, 4096 * (k + 1), k + 1), (2200, 4096 * k, k)]:
+    assert T["drift_fwd_two_tiles_min_rows"] <= 2304
+    for n, L, slots, team in [(2100, 4096 * (k + 1), 2, (k + 1) // 2), (2200, 4096 * k, 1, k), (2304, 16384, 2, 2)]:
         g = torch.Generator().manual_seed(n)
         x, c, dy = (torch.randn(n, L, generator=g), torch.rand(n, L, generator=g), torch.randn(n, L, generator=g))
         xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
         plan = nat.plan(xd, reverse)
-        assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == (nat.FAMILY_DRIFT, 16, 1, team), plan
+        assert (plan["family"], plan["waves"], plan["slots"], plan["tasks"]) == (nat.FAMILY_DRIFT, 16, slots, team), plan
         bwd_family = nat.plan(xd, reverse, True)["family"]
         assert bwd_family == (nat.FAMILY_DRIFT if n <= nat.plan_thresholds()["drift_bwd_max_rows"] else bwd_family)
         assert bwd_family in (nat.FAMILY_SWEEP, nat.FAMILY_STREAM, nat.FAMILY_DRIFT)

@@ -294,8 +294,17 @@ class TestPlanner:
         # the backward of enough rows with at least four such tiles
         assert T["drift_min_small_tiles_per_row"] > 6 and 128 < T["drift_bwd_short_rows_min_rows"] <= 2048
         short_bwd = lambda n: D if n >= T["drift_bwd_short_rows_min_rows"] else ST
+        # (the forward of rows of two tiles of 8192 elements: teams of two from drift_fwd_two_tiles_min_rows rows on)
+        two_fwd = lambda n: D if n >= T["drift_fwd_two_tiles_min_rows"] else ST
         assert [fam(shape, b) for shape in [(2048, 16384), (768, 16384), (400, 24576), (130, 16384)] for b in (False, True)] == \
-            [ST, short_bwd(2048), ST, short_bwd(768), ST, short_bwd(400), ST, short_bwd(130)]
+            [two_fwd(2048), short_bwd(2048), two_fwd(768), short_bwd(768), ST, short_bwd(400), ST, short_bwd(130)]
+        n2 = T["drift_fwd_two_tiles_min_rows"]
+        q = nat.plan(torch.empty(n2, 16384))
+        assert (q["family"], q["waves"], q["slots"], q["tasks"], q["tiles_per_row"]) == (D, 16, 2, 2, 2), q
+        assert fam((n2 - 1, 16384)) == ST and T["drift_fwd_min_tiles_per_row"] >= 2
+        # beyond 2048 rows the forward keeps its tiles of 8192 elements
+        q = nat.plan(torch.empty(4096, 32768))
+        assert (q["family"], q["waves"], q["slots"], q["tasks"]) == (D, 16, 2, 4), q
         n = T["drift_bwd_short_rows_min_rows"]
         # (rows of seven such tiles: enough work in all for the rule on little work in many rows not to apply)
         assert fam((n, 28672), True) == D and fam((n - 1, 28672), True) != D
@@ -306,10 +315,10 @@ class TestPlanner:
         assert fam((96, 65536), True) == W and fam((24, 262144), True) == W
         assert fam((16, 1 << 20), True) == D and fam((100, 131072), True) == D and fam((128, 262144), True) == D
         assert fam((512, 262144), True) == D and fam((256, 262144), True) == D
-        # more than 2048 rows: the forward still, in tiles of 4096 elements; the backward in teams that wait (up to
+        # more than 2048 rows: the forward still, in its tiles of 8192 elements; the backward in teams that wait (up to
         # 1024 rows of 16 tiles and more) or one workgroup per row; ragged rows one workgroup per row
         q = nat.plan(torch.empty(4096, 65536))
-        assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 1, 16, 256), q
+        assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 2, 8, 256), q
         m = T["drift_bwd_max_rows"]
         assert 1024 <= m and fam((m, 65536), True) == D and fam((m + 256, 65536), True) == W
         assert fam((m + 256, 131072), True) == ST and fam((4096, 65536 + 8)) == ST
@@ -320,7 +329,7 @@ class TestPlanner:
         assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
-        assert slots((4000, 24576)) == 4 and slots((838, 40000)) == 4 and slots((800, 36000)) == 2
+        assert slots((700, 24576)) == 4 and slots((838, 40000)) == 4 and slots((800, 36000)) == 2
         assert fam((300, 65536 + 4)) == nat.FAMILY_STREAM          # ragged last tile
         # ... whose rows beyond one per CU, if few, go to a second launch of their own (teams per row)
         p = nat.plan(torch.empty(300, 65536 + 4))
