@@ -45,17 +45,57 @@ __device__ __forceinline__ float read_lane(float v, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
+// One Kogge-Stone step on N (1, 2 or 4) independent rows of pairs, two instructions a row: the multiply-add and the
+// multiply read their first operand through DPP themselves (v_fmac_f32_dpp b, b', a: b += b' * a with b' the source
+// lane's b; v_mul_f32_dpp a, a', a), and a lane without a source, or in a row masked out, is switched off for the
+// instruction and keeps its pair - which is what composing with the identity gives.  The compiler does not fold a
+// v_mov_b32_dpp into the arithmetic here (it leaves two moves that set the identity, two DPP moves, the multiply-add
+// and the multiply: six instructions a row), hence the assembly.  A DPP operand must not be read within two wait
+// states of the vector instruction that wrote it: the leading s_nop covers what the compiler placed in front, inside
+// a block no instruction reads through DPP what the block wrote (the multiply-adds write b, the multiplies read a),
+// and behind the block the compiler pads for its own DPP reads.
+#define LINREC_DPP_FMAC(B, A, MODS) "v_fmac_f32_dpp " B ", " B ", " A " " MODS "\n\t"
+#define LINREC_DPP_MUL(A, MODS) "v_mul_f32_dpp " A ", " A ", " A " " MODS "\n\t"
+#define LINREC_DPP_STEP_ROWS(MODS)                                                                                  \
+  if constexpr (N == 1) {                                                                                           \
+    asm("s_nop 1\n\t" LINREC_DPP_FMAC("%0", "%1", MODS) LINREC_DPP_MUL("%1", MODS) : "+v"(b[0]), "+v"(a[0]));      \
+  } else if constexpr (N == 2) {                                                                                    \
+    asm("s_nop 1\n\t" LINREC_DPP_FMAC("%0", "%2", MODS) LINREC_DPP_FMAC("%1", "%3", MODS)                           \
+        LINREC_DPP_MUL("%2", MODS) LINREC_DPP_MUL("%3", MODS)                                                       \
+        : "+v"(b[0]), "+v"(b[1]), "+v"(a[0]), "+v"(a[1]));                                                          \
+  } else {                                                                                                          \
+    asm("s_nop 1\n\t" LINREC_DPP_FMAC("%0", "%4", MODS) LINREC_DPP_FMAC("%1", "%5", MODS)                           \
+        LINREC_DPP_FMAC("%2", "%6", MODS) LINREC_DPP_FMAC("%3", "%7", MODS) LINREC_DPP_MUL("%4", MODS)              \
+        LINREC_DPP_MUL("%5", MODS) LINREC_DPP_MUL("%6", MODS) LINREC_DPP_MUL("%7", MODS)                            \
+        : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));          \
+  }
+template <int CTRL, int ROW_MASK, int N>
+__device__ __forceinline__ void scan_step_rows(float* a, float* b) {
+  static_assert(N == 1 || N == 2 || N == 4, "rows of one block");
+  static_assert(ROW_MASK == (CTRL == DPP_ROW_BCAST15 ? 0xa : CTRL == DPP_ROW_BCAST31 ? 0xc : 0xf), "row mask of the step");
+  if constexpr (CTRL == DPP_ROW_SHR1) { LINREC_DPP_STEP_ROWS("row_shr:1 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHR2) { LINREC_DPP_STEP_ROWS("row_shr:2 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHR4) { LINREC_DPP_STEP_ROWS("row_shr:4 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHR8) { LINREC_DPP_STEP_ROWS("row_shr:8 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHL1) { LINREC_DPP_STEP_ROWS("row_shl:1 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHL2) { LINREC_DPP_STEP_ROWS("row_shl:2 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHL4) { LINREC_DPP_STEP_ROWS("row_shl:4 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_SHL8) { LINREC_DPP_STEP_ROWS("row_shl:8 row_mask:0xf bank_mask:0xf") }
+  else if constexpr (CTRL == DPP_ROW_BCAST15) { LINREC_DPP_STEP_ROWS("row_bcast:15 row_mask:0xa bank_mask:0xf") }
+  else { static_assert(CTRL == DPP_ROW_BCAST31, "a step of the scan"); LINREC_DPP_STEP_ROWS("row_bcast:31 row_mask:0xc bank_mask:0xf") }
+}
+#undef LINREC_DPP_STEP_ROWS
+#undef LINREC_DPP_MUL
+#undef LINREC_DPP_FMAC
+
 // One Kogge-Stone step on R independent rows of pairs: every lane with a source composes the
-// source's pair in front of its own.  Lanes without a source see the identity.
+// source's pair in front of its own.  Lanes without a source keep theirs.
 template <int CTRL, int ROW_MASK, int R>
 __device__ __forceinline__ void scan_step(float (&a)[R], float (&b)[R]) {
+  constexpr int N = R >= 4 ? 4 : R >= 2 ? 2 : 1;  // rows to a block
+  static_assert(R % N == 0, "whole blocks");
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float pa = dpp_move<CTRL, ROW_MASK>(1.0f, a[r]);
-    float pb = dpp_move<CTRL, ROW_MASK>(0.0f, b[r]);
-    b[r] = fmaf(pb, a[r], b[r]);
-    a[r] = pa * a[r];
-  }
+  for (int r = 0; r < R; r += N) scan_step_rows<CTRL, ROW_MASK, N>(a + r, b + r);
 }
 
 // Inclusive scan over the 64 lanes of R independent rows of affine maps (lane 0 first).
