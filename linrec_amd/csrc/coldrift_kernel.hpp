@@ -34,6 +34,71 @@ struct ColDriftArgs {
   TileArgs chain;  // of it: ws, counters, desc, ws_tiles, spin_limit, num_tiles (workgroups), tasks (team size M)
 };
 
+// What a lane keeps of one position of its VEC rows from the load to the store three steps later: the values as
+// loaded.  16-bit storage stays packed (two rows to a register) and is widened where it is used, so that a step of
+// two rows per lane holds as many registers, and moves as many bytes, as an fp32 step of one.
+template <typename T, int VEC>
+struct Held {
+  using V = typename Pack<T, VEC>::type;
+  V q;
+};
+template <int VEC>
+struct Held<float, VEC> {
+  Lanes<VEC> q;
+};
+template <int VEC, typename T>
+__device__ __forceinline__ Held<T, VEC> ld_held(const T* p) {
+  Held<T, VEC> h;
+  if constexpr (std::is_same_v<T, float>) {
+    h.q = ld_rows<VEC>(p);
+  } else {
+    using V = typename Pack<T, VEC>::type;
+    h.q = stream_load(reinterpret_cast<const V*>(p));
+  }
+  return h;
+}
+template <typename T, int VEC>
+__device__ __forceinline__ Lanes<VEC> widen(const Held<T, VEC>& h) {
+  if constexpr (std::is_same_v<T, float>) {
+    return h.q;
+  } else {
+    Lanes<VEC> r;
+    if constexpr (VEC > 1) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) r.v[e] = float(h.q[e]);
+    } else {
+      r.v[0] = float(h.q);
+    }
+    return r;
+  }
+}
+// The same values as something the compiler knows nothing about: what was widened from `h` before is not what is
+// widened from the result, so the packed register stays the one that lives from a step's scan to its store (the
+// compiler would rather keep the widened values, two registers for one).
+template <typename T, int VEC>
+__device__ __forceinline__ Held<T, VEC> held_again(Held<T, VEC> h) {
+  if constexpr (!std::is_same_v<T, float> && sizeof(typename Pack<T, VEC>::type) == 4) {
+    uint32_t bits = __builtin_bit_cast(uint32_t, h.q);
+    asm volatile("" : "+v"(bits));
+    h.q = __builtin_bit_cast(typename Pack<T, VEC>::type, bits);
+  }
+  return h;
+}
+template <typename T, int VEC>
+__device__ __forceinline__ Held<T, VEC> held_zero() {
+  Held<T, VEC> h;
+  if constexpr (std::is_same_v<T, float> || VEC > 1) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if constexpr (std::is_same_v<T, float>) h.q.v[e] = 0.0f;
+      else h.q[e] = T(0.0f);
+    }
+  } else {
+    h.q = T(0.0f);
+  }
+  return h;
+}
+
 template <typename T, int VEC, int U, int NW, int G, int MODE, bool DESC>
 __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   static_assert(G == 1 || G == 2, "a wave is whole or split into its two halves");
@@ -84,24 +149,23 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   uint64_t* const desc = ch.desc + 2 * (block * ksteps) * RPB;
 
   struct Batch {
-    Lanes<VEC> x[U], c[U], yn[NEED_Y ? U : 1];
+    Held<T, VEC> x[U], c[U], yn[NEED_Y ? U : 1];
   };
-  auto load_batch = [&](Batch& bt, int n0) {
+  auto load_batch = [&](Batch& bt, int n0) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int n = n0 + u;  // position in scan order
       const int l = DESC ? L - 1 - n : n;
       if (n < L) {
         const long long off = base + (long long)l * p.elem_stride;
-        bt.x[u] = ld_rows<VEC>(in0 + off);
-        bt.c[u] = ld_rows<VEC>(coef + off);
+        bt.x[u] = ld_held<VEC>(in0 + off);
+        bt.c[u] = ld_held<VEC>(coef + off);
         if constexpr (NEED_Y) {
           const int ln = DESC ? l - 1 : l + 1;  // saved output one step further along this scan
           if (ln >= 0 && ln < L) {
-            bt.yn[u] = ld_rows<VEC>(aux + base + (long long)ln * p.elem_stride);
+            bt.yn[u] = ld_held<VEC>(aux + base + (long long)ln * p.elem_stride);
           } else {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) bt.yn[u].v[e] = 0.0f;
+            bt.yn[u] = held_zero<T, VEC>();
           }
         }
       }
@@ -124,7 +188,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   struct Words {
     uint64_t w0[VEC], w1[VEC];
   };
-  auto ask = [&](int k, Words& w) {
+  auto ask = [&](int k, Words& w) __attribute__((always_inline)) {
     const int need = k < M - 1 ? k : M - 1;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
@@ -140,10 +204,10 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
       }
     }
   };
-  auto collect = [&](int k, Words w, int slot, int token) {
+  auto collect = [&](int k, Words w, int slot, int token) __attribute__((always_inline)) {
     const int need = k < M - 1 ? k : M - 1;
     if (wave >= need) return;
-    auto all_there = [&]() {
+    auto all_there = [&]() __attribute__((always_inline)) {
       bool have = true;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) have = have && uint32_t(w.w0[e] >> 32) == want && uint32_t(w.w1[e] >> 32) == want;
@@ -175,7 +239,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   };
   // What enters position n_end of this lane's rows, from the rows' own data (when a wait ran out): the
   // plain sequential walk.
-  auto recompute = [&](int n_end) {
+  auto recompute = [&](int n_end) __attribute__((always_inline)) {
     Lanes<VEC> val;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) val.v[e] = 0.0f;
@@ -193,7 +257,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   };
 
   // First half of own step i (tile in D[PH], step k of the row): the lane's map, the waves' maps to LDS.
-  auto scan_step = [&]<int PH>(std::integral_constant<int, PH>, int k) {
+  auto scan_step = [&]<int PH>(std::integral_constant<int, PH>, int k) __attribute__((always_inline)) {
     const Batch& bt = D[PH];
     Pending& now = P[PH];
     const int n0 = k * STEP + run * U;
@@ -207,15 +271,16 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
     for (int u = 0; u < U; ++u) {
       const int n = n0 + u;
       if (n < L) {
+        const Lanes<VEC> x = widen(bt.x[u]), c = widen(bt.c[u]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           if constexpr (MODE == 0) {
             // the coefficient of the first position takes no part (linrec_ref.cuh:63)
-            mb.v[e] = n == 0 ? bt.x[u].v[e] : fmaf(mb.v[e], bt.c[u].v[e], bt.x[u].v[e]);
-            ma.v[e] = n == 0 ? 0.0f : ma.v[e] * bt.c[u].v[e];
+            mb.v[e] = n == 0 ? x.v[e] : fmaf(mb.v[e], c.v[e], x.v[e]);
+            ma.v[e] = n == 0 ? 0.0f : ma.v[e] * c.v[e];
           } else {
-            mb.v[e] = (mb.v[e] + bt.x[u].v[e]) * bt.c[u].v[e];
-            ma.v[e] *= bt.c[u].v[e];
+            mb.v[e] = (mb.v[e] + x.v[e]) * c.v[e];
+            ma.v[e] *= c.v[e];
           }
         }
       }
@@ -241,7 +306,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
     now.k = k;
   };
   // After the barrier of own step i: wave 0 publishes the whole map of the step just scanned.
-  auto publish = [&]<int PH>(std::integral_constant<int, PH>, int k) {
+  auto publish = [&]<int PH>(std::integral_constant<int, PH>, int k) __attribute__((always_inline)) {
     if (wave != 0 || (G > 1 && grp != 0) || k + 1 >= ksteps) return;
     Lanes<VEC> ta, tb;
 #pragma unroll
@@ -267,7 +332,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   };
   // After the barrier: pending step in P[PH] (step k of the row, its waves' maps in sh_a/sh_b[PH]) gets the
   // value that enters it, is walked again from there and stored.
-  auto store_step = [&]<int PH>(std::integral_constant<int, PH>, int slot, int token) {
+  auto store_step = [&]<int PH>(std::integral_constant<int, PH>, int slot, int token) __attribute__((always_inline)) {
     const Pending& q = P[PH];
     const Batch& bt = D[PH];
     const int k = q.k;
@@ -313,17 +378,19 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
       const int l = DESC ? L - 1 - n : n;
       if (n < L) {
         const long long off = base + (long long)l * p.elem_stride;
+        const Lanes<VEC> x = widen(held_again(bt.x[u])), c = widen(held_again(bt.c[u]));
         if constexpr (MODE == 0) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) val.v[e] = n == 0 ? bt.x[u].v[e] : fmaf(val.v[e], bt.c[u].v[e], bt.x[u].v[e]);
+          for (int e = 0; e < VEC; ++e) val.v[e] = n == 0 ? x.v[e] : fmaf(val.v[e], c.v[e], x.v[e]);
           if (active) st_rows<VEC>(out0 + off, val);
         } else {
+          const Lanes<VEC> yn = widen(held_again(bt.yn[u]));
           Lanes<VEC> dx, dc;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
-            dx.v[e] = val.v[e] + bt.x[u].v[e];
-            dc.v[e] = dx.v[e] * bt.yn[u].v[e];
-            val.v[e] = dx.v[e] * bt.c[u].v[e];
+            dx.v[e] = val.v[e] + x.v[e];
+            dc.v[e] = dx.v[e] * yn.v[e];
+            val.v[e] = dx.v[e] * c.v[e];
           }
           if (active) {
             st_rows<VEC>(out0 + off, dx);
@@ -336,7 +403,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
 
   // Own step i, i % 4 == PH: step k = j + i * M of the row lies in D[PH]; D[(PH + 2) % 4] is own step i - 2,
   // stored in this step; D[(PH + 1) % 4] takes the loads of own step i + 1.
-  auto step = [&]<int PH>(std::integral_constant<int, PH> ph, int i) {
+  auto step = [&]<int PH>(std::integral_constant<int, PH> ph, int i) __attribute__((always_inline)) {
     constexpr int OLD = (PH + 2) % 4, LD = (PH + 1) % 4;
     const int k = j + i * M;
     __builtin_amdgcn_sched_barrier(0);  // (nothing of this step moves up into the one before)
@@ -353,7 +420,7 @@ __global__ __launch_bounds__(64 * NW) void coldrift_kernel(ColDriftArgs args) {
   };
   // The last step lies in D[A] and the one before it in D[(A + 3) % 4]: nothing left to overlap with, so
   // both are asked for at once, and one barrier serves both.
-  auto finish = [&]<int A>(std::integral_constant<int, A>) {
+  auto finish = [&]<int A>(std::integral_constant<int, A>) __attribute__((always_inline)) {
     constexpr int PREV = (A + 3) % 4;
     Words w, v;
     if (own >= 2) ask(P[PREV].k, w);

@@ -174,7 +174,8 @@ KernelGroup kernels_bf16_cols();
   GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
   COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16), \
   SEGMENT_(TY, 4, 8), SEGMENT_(TY, 2, 8), SEGMENT_(TY, 1, 8),                                   \
-  COLBLOCK_FWD_(TY, 2, 8, 1), COLBLOCK_BWD_(TY, 2, 4, 1), COLBLOCK_FWD_(TY, 2, 8, 2), COLBLOCK_BWD_(TY, 2, 4, 2)
+  COLBLOCK_FWD_(TY, 2, 8, 1), COLBLOCK_BWD_(TY, 2, 4, 1), COLBLOCK_FWD_(TY, 2, 8, 2), COLBLOCK_BWD_(TY, 2, 4, 2), \
+  COLDRIFT_FWD_(TY, 16, 2, 8), COLDRIFT_BWD_(TY, 8, 2, 16), COLDRIFT_FWD_(TY, 8, 2, 16), COLDRIFT_BWD_(TY, 16, 2, 4)
 
 #define LINREC_KERNEL_GROUP(NAME, ...)                                                          \
   namespace linrec {                                                                            \

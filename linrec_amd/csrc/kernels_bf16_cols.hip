@@ -5,6 +5,7 @@
 #include "flat_kernel.hpp"
 #include "column_kernel.hpp"
 #include "colblock_kernel.hpp"
+#include "coldrift_kernel.hpp"
 #include "kernel_table.hpp"
 
 LINREC_KERNEL_GROUP(kernels_bf16_cols,

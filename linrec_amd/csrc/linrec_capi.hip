@@ -521,44 +521,6 @@ int colblock_kernel_for(const Problem& q, int vec, int groups, int want_depth, i
   }
   return -1;
 }
-// Column drift kernels: the team size for `blocks` blocks of rows of `steps` steps each, 0 if the launch
-// would not be worth it: the power of two that fills the chip, every member with at least four steps.
-int64_t coldrift_team(const Problem& q, int64_t blocks, int64_t steps, int64_t resident, int waves) {
-  int64_t team = 1;
-  while (team * 2 <= waves && blocks * team * 2 <= resident && steps >= 8 * team) team *= 2;
-  return team >= 2 && blocks * team * 2 > q.cus ? team : 0;
-}
-// Whether the planner gives this problem (strided scan axis) to the column drift kernels: fp32 rows next to
-// each other, few enough that teams of at least 4 (backward: 2) along the scan axis are what fills the chip,
-// and enough of them that the teams fill three quarters of it.  Measured forward / backward in us against
-// what the table chose before (segments up to 4095 rows, column blocks from there): 4096 x 16384 157.1 / 255.5
-// against 216.3 / 307.1; 2048 x 16384 83.6 / 132.0 against 107.4 / 150.4; 1024 x 32768 forward 95.6 against
-// 110.4 (backward 162.1 against 154.6: left to the segments); 8192 x 4096 backward 126.8 against 142.7 (forward
-// 80.5 against 78.9: left to the column blocks); 3072 x 16384 140.5 / 213.5 against 168.4 / 248.2; 2048 x 4096
-// 25.5 / 36.2 against 40.8 / 54.3; 4096 x 2048 24.9 / 34.3 against 29.5 / 47.7; 512 x 65536 161.3 / 284.5
-// against 112.7 / 149.9 (left to the segments).
-bool coldrift_applies(const Problem& q) {
-  if (q.dtype != LINREC_DTYPE_F32 || q.seqlen < 2048) return false;
-  if (q.row_stride != 1 && q.numseq != 1 && q.rows_per_batch != 1) return false;
-  const int waves = q.is_bwd ? 8 : 16;
-  const int64_t blocks = ceil_div(q.numseq, 64);
-  const int64_t steps = ceil_div(q.seqlen, 128);
-  const int64_t team = coldrift_team(q, blocks, steps, q.cus, waves);
-  // (a caller that can only give so much workspace is served by the kernels that need less)
-  if (q.workspace_cap && linrec_workspace_bytes_for_tiles(blocks * steps * 64) > q.workspace_cap) return false;
-  // Teams of 16 only where they fill seven eighths of the chip: 768 x 32768 forward 91.4 us in 192 workgroups
-  // against 82.6 us for the segments, 900 x 32768 97.6 us in 240 against 117.6 us, 1024 x 32768 98.7 against
-  // 109.1 us.  Teams of 2, which gain least, only where they fill it: 6144 x 4096 backward 110.6 us in 192
-  // workgroups against 108.3 us for the column blocks, 8192 x 4096 127.3 against 141.0 us.  Teams of 4 and 8 from
-  // 65 % on, forward / backward: 1300 x 16384 in 168 workgroups 76.4 / 116.8 us against 86.4 / 128.3 us, 3000 x 8000
-  // in 188 80.5 / 132.0 us against 93.7 / 131.0 us; 2560 x 8192 in 160 70.3 / 102.4 us against 69.5 / 97.7 us,
-  // 1100 x 16384 in 144 74.3 / 107.8 us against 75.7 / 109.9 us, 2200 x 16384 in 140 141.5 / 216.0 us against
-  // 134.9 / 199.6 us.
-  if (team < (q.is_bwd ? 2 : 4)) return false;
-  if (team == 2) return blocks * team >= q.cus;
-  if (team > 8) return blocks * team * 8 >= 7 * q.cus;
-  return blocks * team * 20 >= 13 * q.cus;
-}
 // Rows per lane (`want`, or the planner's choice for 0) if the layout allows a block kernel, else 0.
 int colblock_rows_per_lane(const Problem& q, int want) {
   if (q.elem_stride == 1 && q.seqlen != 1) return 0;
@@ -576,6 +538,63 @@ int colblock_rows_per_lane(const Problem& q, int want) {
   return v;
 }
 
+// Column drift kernels: the team size for `blocks` blocks of rows of `steps` steps each, 0 if the launch
+// would not be worth it: the power of two that fills the chip, every member with at least four steps.
+// 16-bit storage (blocks of 128 rows, two to a lane): teams of 4 or 8, every member with at least two steps (bf16
+// 4096 x 2048 in teams of 8: 18.1 / 22.7 us against 28.4 / 38.4 us for the segments).
+int64_t coldrift_team(const Problem& q, int64_t blocks, int64_t steps, int64_t resident, int waves) {
+  int64_t team = 1;
+  if (q.dtype != LINREC_DTYPE_F32) {
+    while (team * 2 <= 8 && blocks * team * 2 <= resident && steps >= 4 * team) team *= 2;
+    return team >= 4 ? team : 0;
+  }
+  while (team * 2 <= waves && blocks * team * 2 <= resident && steps >= 8 * team) team *= 2;
+  return team >= 2 && blocks * team * 2 > q.cus ? team : 0;
+}
+// Whether the planner gives this problem (strided scan axis) to the column drift kernels: fp32 rows next to
+// each other, few enough that teams of at least 4 (backward: 2) along the scan axis are what fills the chip,
+// and enough of them that the teams fill three quarters of it.  Measured forward / backward in us against
+// what the table chose before (segments up to 4095 rows, column blocks from there): 4096 x 16384 157.1 / 255.5
+// against 216.3 / 307.1; 2048 x 16384 83.6 / 132.0 against 107.4 / 150.4; 1024 x 32768 forward 95.6 against
+// 110.4 (backward 162.1 against 154.6: left to the segments); 8192 x 4096 backward 126.8 against 142.7 (forward
+// 80.5 against 78.9: left to the column blocks); 3072 x 16384 140.5 / 213.5 against 168.4 / 248.2; 2048 x 4096
+// 25.5 / 36.2 against 40.8 / 54.3; 4096 x 2048 24.9 / 34.3 against 29.5 / 47.7; 512 x 65536 161.3 / 284.5
+// against 112.7 / 149.9 (left to the segments).
+//
+// 16-bit storage, two rows to a lane (four bytes' worth, as fp32's one): the teams are twice as large for the same rows,
+// so they pay where teams of 4 fill three quarters of the chip and teams of 8 seven eighths of it.  bf16, forward /
+// backward in us against the table's choice before (segments; column blocks for the forward of 8192 rows): 4096 x 16384
+// in teams of 8 108.3 / 156.1 against 130.9 / 164.4, 8192 x 4096 in teams of 4 52.0 / 78.5 against 63.3 / 93.3, 6144 x
+// 4096 (192 workgroups) 46.3 / 68.3 against 55.9 / 73.9, 4096 x 2048 18.1 / 22.7 against 28.4 / 38.4; but 3072 x 16384
+// (teams of 8 in 192 workgroups) 100.9 / 142.1 against 96.4 / 127.1, 2560 x 8192 50.8 / 71.3 against 48.2 / 64.5, and
+// teams of 16 (2048 x 16384: 67.7 / 122.2 against 66.4 / 92.2; 2048 x 4096 21.9 / 31.3 against 26.9 / 36.5) or of 2
+// (16384 x 4096: 96.3 / 145.6 against 79.4 / 132.8 for the column blocks) are left out.
+bool coldrift_applies(const Problem& q) {
+  const bool half = q.dtype != LINREC_DTYPE_F32;
+  if (q.seqlen < 2048) return false;
+  if (q.row_stride != 1 && q.numseq != 1 && q.rows_per_batch != 1) return false;
+  const int vec = half ? 2 : 1;
+  if (colblock_rows_per_lane(q, vec) != vec) return false;
+  const int waves = q.is_bwd ? 8 : 16;
+  const int64_t blocks = ceil_div(ceil_div(q.numseq, vec), 64);
+  const int64_t steps = ceil_div(q.seqlen, 128);
+  const int64_t team = coldrift_team(q, blocks, steps, q.cus, waves);
+  // (a caller that can only give so much workspace is served by the kernels that need less)
+  if (q.workspace_cap && linrec_workspace_bytes_for_tiles(blocks * steps * 64 * vec) > q.workspace_cap) return false;
+  if (half) return team == 4 ? blocks * team * 4 >= 3 * q.cus : team == 8 && blocks * team * 8 >= 7 * q.cus;
+  // Teams of 16 only where they fill seven eighths of the chip: 768 x 32768 forward 91.4 us in 192 workgroups
+  // against 82.6 us for the segments, 900 x 32768 97.6 us in 240 against 117.6 us, 1024 x 32768 98.7 against
+  // 109.1 us.  Teams of 2, which gain least, only where they fill it: 6144 x 4096 backward 110.6 us in 192
+  // workgroups against 108.3 us for the column blocks, 8192 x 4096 127.3 against 141.0 us.  Teams of 4 and 8 from
+  // 65 % on, forward / backward: 1300 x 16384 in 168 workgroups 76.4 / 116.8 us against 86.4 / 128.3 us, 3000 x 8000
+  // in 188 80.5 / 132.0 us against 93.7 / 131.0 us; 2560 x 8192 in 160 70.3 / 102.4 us against 69.5 / 97.7 us,
+  // 1100 x 16384 in 144 74.3 / 107.8 us against 75.7 / 109.9 us, 2200 x 16384 in 140 141.5 / 216.0 us against
+  // 134.9 / 199.6 us.
+  if (team < (q.is_bwd ? 2 : 4)) return false;
+  if (team == 2) return blocks * team >= q.cus;
+  if (team > 8) return blocks * team * 8 >= 7 * q.cus;
+  return blocks * team * 20 >= 13 * q.cus;
+}
 // The rows a second launch serves: the last `tail_rows` rows of `q`, as a problem of their own.
 Problem tail_problem(const Problem& q, int64_t tail_rows) {
   Problem t = q;
@@ -983,7 +1002,8 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
   // `slots` = positions per run, `carry` = rows per lane, `tasks` = team size).
   if (family == LINREC_FAMILY_COLDRIFT) {
     const bool given = tune && tune->family == LINREC_FAMILY_COLDRIFT;
-    const int vec = colblock_rows_per_lane(q, given && tune->carry > 0 ? tune->carry : 1);
+    // (a lane takes four bytes' worth of rows: a wave reads 256 bytes of every position)
+    const int vec = colblock_rows_per_lane(q, given && tune->carry > 0 ? tune->carry : half ? 2 : 1);
     if (vec == 0) return LINREC_E_UNSUPPORTED;
     int waves = 0, depth = 0, id = -1;
     // (waves, positions per run) in the planner's order of preference: forward 16 waves with runs of 8;

@@ -86,7 +86,7 @@ def candidates(t):
             for groups in (1, 2):
                 out.append((f"column block rows {width} groups {groups}", nat.Tuning(nat.FAMILY_COLUMN, width, 0, groups)))
         # column blocks in teams along the scan axis: waves per workgroup, positions per run, rows per lane, team size
-        for w, run, width in ((16, 8, 1), (16, 4, 1), (8, 16, 1)):
+        for w, run, width in ((16, 8, 1), (16, 4, 1), (8, 16, 1), (16, 8, 2), (16, 4, 2), (8, 16, 2)):  # (two rows per lane: 16-bit storage)
             out.append((f"column drift w{w} run {run} rows {width}", nat.Tuning(nat.FAMILY_COLDRIFT, w, run, width)))
             for team in (2, 4, 8, 16):
                 out.append((f"column drift w{w} run {run} rows {width} x{team}", nat.Tuning(nat.FAMILY_COLDRIFT, w, run, width, team)))

@@ -238,3 +238,76 @@ def _poll_limit_one(nat, shape, dtype, reverse):
     dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y_kept.cpu()), reverse)
     _check(dx, dx_t, dtype, "d_inputs with a poll limit of one")
     _check(dc, dc_t, dtype, "d_coeffs with a poll limit of one")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_column_drift_kernels_two_rows_per_lane(nat, reverse, dtype):
+    """Scan axis strided, 16-bit storage: blocks of 128 rows (two to a lane, kept packed from a step's loads to its
+    stores) in teams along the scan axis.  Every compiled geometry is forced with team sizes from 1 to 8 on row lengths
+    around whole steps, on fewer steps than team members allow and on row counts that leave lanes without rows; then
+    the planner's own choice, a batch of time-major matrices, and a poll limit of one."""
+    D = nat.FAMILY_COLDRIFT
+    dev = torch.device("cuda:0")
+    f64 = lambda t: t.float().numpy().astype(np.float64)
+    for n, L in [(128, 256), (2, 129), (130, 257), (66, 1000), (1000, 1290), (190, 2048), (4100, 700)]:
+        x, c, dy = _inputs((n, L), dtype, n + L, transposed=True)
+        y_kept = None
+        for waves, run, passes in [(16, 8, "f"), (8, 16, "fb"), (16, 4, "b")]:
+            steps, blocks = -(-L // (waves * run)), -(-(n // 2) // 64)
+            for team in sorted({1, 2, 3, min(waves, steps), min(8, steps)}):
+                if team > steps or blocks * team > 256:
+                    continue
+                tuning = nat.Tuning(D, waves, run, 2, team)
+                label = f"{dtype} rev={reverse} {n} x {L} waves={waves} run={run} team={team}"
+                plan = nat.plan(x.to(dev), reverse, passes == "b", tuning)
+                assert (plan["family"], plan["vec"], plan["block"], plan["tasks"], plan["grid"], plan["tiles_per_row"]) == (
+                    D, 2, 64 * waves, team, blocks * team, steps), plan
+                if passes != "b":
+                    _run(nat, x, c, dy, reverse, tuning, label, backward_too=passes == "fb")
+                else:
+                    if y_kept is None:
+                        y_kept = nat.fwd(x.to(dev), c.to(dev), reverse)
+                    dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y_kept.cpu()), reverse)
+                    dx, dc = nat.bwd(dy.to(dev), c.to(dev), y_kept, reverse, tuning, out=(_nan_like(y_kept), _nan_like(y_kept)))
+                    torch.cuda.synchronize()
+                    _check(dx, dx_t, dtype, label + " d_inputs")
+                    _check(dc, dc_t, dtype, label + " d_coeffs")
+                    assert nat.gave_up_count() == 0
+    # the planner's own choice, both passes: teams of 8 on 4096 rows
+    x, c, dy = _inputs((4096, 2100), dtype, 5, transposed=True, coeffs="near1")
+    for is_bwd in (False, True):
+        plan = nat.plan(x.to(dev), reverse, is_bwd)
+        assert (plan["family"], plan["vec"], plan["tasks"], plan["grid"]) == (D, 2, 8, 256), plan
+    _run(nat, x, c, dy, reverse, None, f"{dtype} transposed 4096 x 2100")
+    # a batch of time-major matrices: 3 x (2100 timesteps x 2688 channels) scanned over time
+    g = torch.Generator().manual_seed(11)
+    xb, cb, dyb = (f((3, 2100, 2688), generator=g).to(dtype) for f in (torch.randn, torch.rand, torch.randn))
+    xv, cv, dyv = (t.to(dev).transpose(1, 2) for t in (xb, cb, dyb))
+    plan = nat.plan(xv, reverse, False)
+    assert plan["family"] == D and plan["grid"] == 63 * plan["tasks"], plan
+    y = nat.fwd(xv, cv, reverse)
+    dx, dc = nat.bwd(dyv, cv, y, reverse)
+    torch.cuda.synchronize()
+    xt, ct, dyt = (t.transpose(1, 2) for t in (xb, cb, dyb))
+    _check(y, oracle.fwd(f64(xt), f64(ct), reverse), dtype, "batched outputs")
+    dx_t, dc_t = oracle.bwd(f64(dyt), f64(ct), f64(y.cpu()), reverse)
+    _check(dx, dx_t, dtype, "batched d_inputs")
+    _check(dc, dc_t, dtype, "batched d_coeffs")
+    # a poll limit of one: waits run out, the value entering a step comes from the rows' own data instead
+    x, c, dy = _inputs((700, 6000), dtype, 3, transposed=True)
+    y_kept = nat.fwd(x.to(dev), c.to(dev), reverse)
+    old = nat.lib().linrec_set_spin_limit(1)
+    try:
+        y = nat.fwd(x.to(dev), c.to(dev), reverse, nat.Tuning(D, 16, 8, 2, 8))
+        dx, dc = nat.bwd(dy.to(dev), c.to(dev), y_kept, reverse, nat.Tuning(D, 8, 16, 2, 8))
+        torch.cuda.synchronize()
+    finally:
+        nat.lib().linrec_set_spin_limit(old)
+    print("16-bit column drift, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
+    for ws in list(nat._workspaces.values()):
+        ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
+    _check(y, oracle.fwd(f64(x), f64(c), reverse), dtype, "poll limit 1 outputs")
+    dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y_kept.cpu()), reverse)
+    _check(dx, dx_t, dtype, "poll limit 1 d_inputs")
+    _check(dc, dc_t, dtype, "poll limit 1 d_coeffs")

@@ -420,8 +420,8 @@ class TestPlanner:
         assert (p["family"], p["vec"], p["slots"]) == (C, 2, 16)
         assert plan(100001, 1024, dtype=torch.float16)["vec"] == 1
         assert plan(1001, 5000)["vec"] == 1 and plan(1001, 5000)["family"] == S
-        p = plan(4096, 16384, dtype=torch.bfloat16)
-        assert (p["family"], p["vec"], p["tiles_per_row"]) == (S, 4, 64)
+        p = plan(2048, 16384, dtype=torch.bfloat16)
+        assert (p["family"], p["vec"], p["tiles_per_row"]) == (S, 4, 128)
         p = nat.plan(torch.empty(16384, 4096).t(), tuning=nat.Tuning(S, 4, 8, -1, 16))
         assert (p["vec"], p["tiles_per_row"], p["tasks"]) == (4, 16, 1024)
         # rows further apart than one element stay with the element-wise kernel
@@ -451,7 +451,23 @@ class TestPlanner:
                 assert names[p["kernel_id"]] == f"coldrift_w{waves}_v1_u{run}_MODE_{'BWD' if bwd else 'FWD'}_{int(bwd)}"
                 # a descriptor of two 64-bit words per row and step, in the lower half of the workspace
                 assert p["workspace_bytes"] >= 2 * 16 * -(-n // 64) * 64 * p["tiles_per_row"]
-        assert plan(4096, 16384, dtype=torch.bfloat16)["family"] == S   # fp32 only
+        # 16-bit storage: two rows to a lane (blocks of 128 rows), teams of 4 from three quarters of the chip on and
+        # teams of 8 from seven eighths on, every member with two steps at least
+        for dtype, pfx in ((torch.bfloat16, "bf16_"), (torch.float16, "f16_")):
+            for n, L, team in [(4096, 16384, 8), (8192, 4096, 4), (6144, 4096, 4), (4096, 2048, 8), (3600, 16384, 8),
+                               (3072, 16384, 0), (2560, 8192, 0), (2048, 16384, 0), (2048, 4096, 0), (16384, 4096, 0),
+                               (1024, 32768, 0), (4097, 16384, 0), (4096, 2000, 0), (5120, 4096, 0)]:
+                for bwd in (False, True):
+                    p = plan(n, L, bwd, dtype=dtype)
+                    if not team:
+                        assert p["family"] in (S, C), (n, L, bwd, p)
+                        continue
+                    waves, run = (8, 16) if bwd else (16, 8)
+                    assert (p["family"], p["waves"], p["slots"], p["vec"], p["tasks"]) == (D, waves, run, 2, team), (n, L, bwd, p)
+                    assert p["grid"] == -(-n // 128) * team <= 256 and p["block"] == 64 * waves
+                    assert p["tiles_per_row"] == -(-L // 128) >= 2 * team
+                    assert names[p["kernel_id"]] == f"{pfx}coldrift_w{waves}_v2_u{run}_MODE_{'BWD' if bwd else 'FWD'}_{int(bwd)}"
+                    assert p["workspace_bytes"] >= 2 * 16 * -(-n // 128) * 128 * p["tiles_per_row"]
         # on request: any compiled geometry, teams of at most as many members as the workgroup has waves
         x = torch.empty(5000, 700).t()
         p = nat.plan(x, tuning=nat.Tuning(D, 8, 16, 1, 4))
@@ -461,6 +477,13 @@ class TestPlanner:
         for bad in (nat.Tuning(D, 8, 16, 1, 16), nat.Tuning(D, 16, 8, 1, 32), nat.Tuning(D, 16, 16, 1, 2), nat.Tuning(D, 16, 8, 2, 2)):
             with pytest.raises(NotImplementedError):
                 nat.plan(x, tuning=bad)
+        xh = torch.empty(5000, 700, dtype=torch.bfloat16).t()
+        p = nat.plan(xh, tuning=nat.Tuning(D, 8, 16, 2, 4))   # 16-bit storage: two rows to a lane, or one on request
+        assert (p["family"], p["vec"], p["grid"], p["tiles_per_row"]) == (D, 2, 6 * 4, 40)
+        with pytest.raises(NotImplementedError):
+            nat.plan(xh, tuning=nat.Tuning(D, 8, 16, 1, 4))
+        with pytest.raises(NotImplementedError):
+            nat.plan(torch.empty(5000, 701, dtype=torch.bfloat16).t(), tuning=nat.Tuning(D, 8, 16, 2, 4))  # an odd number of rows
         with pytest.raises(NotImplementedError):
             nat.plan(torch.empty(700, 5000), tuning=nat.Tuning(D))  # rows along the unit-stride axis
 
