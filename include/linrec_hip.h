@@ -79,9 +79,9 @@ extern "C" {
                                    of workgroups share a block of rows and take its steps along the scan axis in
                                    turn; a step's data stays in registers and is stored two steps late, when the
                                    team mates' maps have arrived.  Tuning: `waves` = waves per workgroup (16 or 8),
-                                   `slots` = positions per run, `carry` = rows per lane, `tasks` = team size (at
-                                   most the waves).  In the plan, `tiles_per_row` = steps of a row, `tasks` = team
-                                   size */
+                                   `slots` = positions per run, `carry` = rows per lane (fp32 one, 16-bit storage
+                                   two), `tasks` = team size (at most the waves).  In the plan, `tiles_per_row` =
+                                   steps of a row, `tasks` = team size */
 
 /*
  * Per-call tuning override; NULL selects the built-in gfx950 table.
