@@ -137,7 +137,9 @@ def test_standalone_driver(extra):
     assert out.returncode == 0, out.stderr
     line = [l for l in out.stdout.splitlines() if l.startswith("max abs difference")][0]
     errs = [float(tok.rstrip(",")) for tok in line.replace(",", " ").split() if "e-" in tok or "e+" in tok]
-    assert len(errs) == 3 and max(errs) < 1e-3, out.stdout
+    # (fp32 against fp32 in another order of operations: values reach about 10, gradients of the coefficients about 30,
+    # so one unit in the last place is 1e-6 to 4e-6; observed 1e-6 / 1e-6 / 3e-6 to 6e-6)
+    assert len(errs) == 3 and max(errs) < 2e-5, out.stdout
     assert "look-backs given up 0" in out.stdout or "workspace 0 bytes" in out.stdout
 
 
