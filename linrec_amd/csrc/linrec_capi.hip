@@ -183,6 +183,7 @@ constexpr int kNumPlanThresholds = int(sizeof(kPlanThresholds) / sizeof(kPlanThr
 
 constexpr int64_t kStreamMinRows = kT_stream_min_rows;   // (these three on 256 CUs; scaled by Problem::at)
 constexpr int64_t kSplitBelowRows = 192;  // rows of a few thousand elements are cut into look-back tiles below this
+                                          // (launches of a few microseconds: the tuning sweep, which times launches from the host, cannot tell them apart)
 constexpr int64_t kSweepBelowRows = 192;  // sweep kernels take 16 .. 191 rows, stream kernels 192 .. 256
 // Fewer long rows: teams of workgroups per row, sized so that at most one workgroup per CU runs
 // (measured at 2^24 elements, forward: 128 rows x2 38 us, 64 x4 39 us, 32 x8 40 us, 16 x16 42 us,
@@ -405,10 +406,10 @@ constexpr int64_t kTailMaxRows = 96;  // rows beyond one per CU that a second la
 constexpr int64_t kGroupMaxSlots = 32;  // rows up to this many slots are packed several to a wave
 constexpr int64_t kTeamMinRows = kT_team_min_rows;
 // 16-bit storage, forward: teams of 64 already win from three rows on (bf16 3 x 4194304 28.0 against 40.3 us for
-// look-back tiles, 4 x 8388608 55.1 against 85.6 us, 5 x 2097152 21.7 against 35.0 us; the backward is a tie:
-// 3 x 4194304 48.7 against 46.4 us, 4 x 8388608 103.7 against 100.1 us)
-constexpr int64_t kTeamMinRowsHalfFwd = 3;
-constexpr int64_t kTeamMinRowsHalfBwd = 6;
+// look-back tiles, 4 x 8388608 55.1 against 85.6 us, 5 x 2097152 21.7 against 35.0 us); the backward from eight (6 x
+// 1048584 25.1 against 19.4 us for look-back tiles, 8 rows 26.2 against 29.5 us).  Both from the generated table.
+constexpr int64_t kTeamMinRowsHalfFwd = kT_half_team_fwd_min_rows;
+constexpr int64_t kTeamMinRowsHalfBwd = kT_half_team_bwd_min_rows;
 
 // Rows one lane of a column kernel takes: 8 bytes' worth (measured best on 262144 x 256: fp32 two
 // rows 131 / 220 us against 132 / 236 us for four; bf16 four rows 70 / 114 us against 101 / 146 us

@@ -330,6 +330,14 @@ CROSSOVERS = [
               lambda v: (v, 16384), [_both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_SWEEP, 8, 2))], _DRIFT,
               passes=("fwd",)),
     # 16-bit storage (measured on bf16; fp16 moves the same bytes)
+    Crossover("half_team_fwd_min_rows", "bf16 forward of a few ragged very long rows (1048584 elements): look-back tiles "
+              "against one team of 64 workgroups per row, by the number of rows", [2, 3, 4, 6, 8, 16, 32],
+              lambda v: (v, 1048584), _both(_t(nat.FAMILY_TILE, 8, 4, 1, 1)), _both(_t(nat.FAMILY_TEAM)), passes=("fwd",),
+              dtype=torch.bfloat16),
+    Crossover("half_team_bwd_min_rows", "bf16 backward of a few ragged very long rows (1048584 elements): look-back tiles "
+              "against one team of 64 workgroups per row, by the number of rows", [2, 3, 4, 6, 8, 16, 32],
+              lambda v: (v, 1048584), _both(_t(nat.FAMILY_TILE, 8, 4, 1, 1)), _both(_t(nat.FAMILY_TEAM)), passes=("bwd",),
+              dtype=torch.bfloat16),
     Crossover("half_drift_fwd_small_tiles_max_rows", "bf16 forward of rows that are whole tiles of 8192 elements but not "
               "of 16384 (nine tiles): drift teams against one workgroup per row, or sweep teams, by the number of rows",
               [64, 96, 112, 127, 144, 160, 200, 256], lambda v: (v, 8192 * 9), _DRIFT_SMALL,
