@@ -63,12 +63,8 @@ __device__ __forceinline__ Lanes<VEC> widen(const Held<T, VEC>& h) {
     return h.q;
   } else {
     Lanes<VEC> r;
-    if constexpr (VEC > 1) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) r.v[e] = float(h.q[e]);
-    } else {
-      r.v[0] = float(h.q);
-    }
+    for (int e = 0; e < VEC; ++e) r.v[e] = float(h.q[e]);
     return r;
   }
 }
@@ -87,14 +83,10 @@ __device__ __forceinline__ Held<T, VEC> held_again(Held<T, VEC> h) {
 template <typename T, int VEC>
 __device__ __forceinline__ Held<T, VEC> held_zero() {
   Held<T, VEC> h;
-  if constexpr (std::is_same_v<T, float> || VEC > 1) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      if constexpr (std::is_same_v<T, float>) h.q.v[e] = 0.0f;
-      else h.q[e] = T(0.0f);
-    }
-  } else {
-    h.q = T(0.0f);
+  for (int e = 0; e < VEC; ++e) {
+    if constexpr (std::is_same_v<T, float>) h.q.v[e] = 0.0f;
+    else h.q[e] = T(0.0f);
   }
   return h;
 }
