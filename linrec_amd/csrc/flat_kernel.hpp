@@ -7,7 +7,8 @@
 // the definition uses no coefficient anyway (linrec/impl/cuda/linrec_ref.cuh:63,
 // linrec/impl/python/ops.py:16-18).  The cut is a flag that travels with the affine maps (a
 // segmented scan), not a multiplication by zero: nothing of a row, non-finite values included,
-// reaches the next one.  A lane computes elements of two or three rows and stores whole slots.
+// reaches the next one.  A lane computes elements of two or three rows - of up to VEC rows where a row is
+// shorter than a slot - and stores whole slots.
 //
 // A wave takes 64 * S consecutive slots (S rows of 64 slots, lanes interleaved for coalescing) and
 // never talks to another wave: what enters its chunk depends on the elements back to the last
@@ -16,7 +17,7 @@
 // whatever came before irrelevant.  No LDS, no barrier, no workspace.
 //
 // Requirements (the planner's): unit element stride, row stride == row length, all bases 16-byte
-// aligned, VEC <= row length <= 64 * VEC.
+// aligned, 2 <= row length <= 64 * VEC.
 //
 // The reference has no counterpart: its kernels give a block to every row
 // (linrec/impl/cuda/linrec_tile.cuh:11-95).
@@ -121,11 +122,15 @@ __global__ __launch_bounds__(256) void flat_kernel(FlatArgs p) {
       if constexpr (MODE == 1) {
         if (j > 0) load_slot_full<VEC, DESC>(aux + s * VEC, 0u, ys);
       }
+      // row positions of the slot's elements in memory order (a row may be shorter than the slot)
+      int rpos[VEC];
+      rpos[0] = r0;
+#pragma unroll
+      for (int e = 1; e < VEC; ++e) rpos[e] = rpos[e - 1] + 1 == L ? 0 : rpos[e - 1] + 1;
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
         const int e = DESC ? VEC - 1 - i : i;  // memory offset inside the slot of scan element i
-        int r = r0 + e;
-        if (r >= L) r -= L;
+        const int r = rpos[e];
         const bool beyond = s * VEC + e >= p.total;  // the tail of the tensor's last slot
         if (beyond) {
           xs[j][i] = 0.0f;

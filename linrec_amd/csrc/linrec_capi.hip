@@ -437,10 +437,10 @@ constexpr int64_t kSegmentMaxSegments = 4096; // (the maps of a row are then 32 
 size_t segment_maps_bytes(int64_t numseq, int64_t segments) { return size_t(2) * size_t(segments) * size_t(numseq) * 4; }
 
 // Flat kernels: dense rows (no gaps between them, so the tensor is one array), every base 16-byte
-// aligned, rows of at least one slot and short enough for one row of 64 slots to look behind.
+// aligned, rows short enough for one row of 64 slots to look behind.
 bool flat_applies(const Problem& q, int fv) {
   return q.elem_stride == 1 && q.numseq > 1 && q.row_stride == q.seqlen && q.base_mis == 0 && !q.batched() &&
-         q.seqlen >= fv && q.seqlen <= 60 * fv;
+         q.seqlen >= 2 && q.seqlen <= 60 * fv;
 }
 // Where they are chosen: up to 40 slots per row.  The look-behind row costs loads in proportion to the
 // row length (2^25 elements, forward / backward: rows of 5 floats 69 / 111 us against 135 / 232 us for

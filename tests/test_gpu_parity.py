@@ -1016,14 +1016,14 @@ def test_short_rows_packed_several_to_a_wave(nat, reverse, dtype):
 @pytest.mark.parametrize("reverse", [False, True])
 def test_dense_short_rows_scanned_as_one_flat_array(nat, reverse, dtype):
     """Dense rows that are not whole 16-byte slots: the flat kernels scan the tensor as one array cut at
-    the row starts.  Row lengths from one slot to sixty, row counts that leave the last slot, the last
-    wave and the look-behind row partly empty, both chunk sizes."""
+    the row starts.  Row lengths from two elements (several rows to a slot) to sixty slots, row counts that leave the
+    last slot, the last wave and the look-behind row partly empty, both chunk sizes."""
     dev = torch.device("cuda:0")
     ve = 4 if dtype == torch.float32 else 8
     tol = TOL_NORMWISE if dtype == torch.float32 else 1.05 * 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
     f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
     F = nat.FAMILY_FLAT
-    for L in [ve, ve + 1, 2 * ve - 1, 3 * ve + 2, 7 * ve + 3, 16 * ve + 1, 33 * ve - 1, 40 * ve - 1, 60 * ve - 3]:
+    for L in [2, 3, ve - 1, ve, ve + 1, 2 * ve - 1, 3 * ve + 2, 7 * ve + 3, 16 * ve + 1, 33 * ve - 1, 40 * ve - 1, 60 * ve - 3]:
         for numseq in [2, 3, 17, 257, 1000, 4099]:
             if numseq * L > 600000:
                 continue

@@ -548,20 +548,21 @@ class TestPlanner:
 
     def test_dense_short_rows_that_are_not_whole_slots_are_scanned_as_one_flat_array(self):
         F, G = nat.FAMILY_FLAT, nat.FAMILY_GROUP
-        for L, slots in [(5, 2), (30, 2), (63, 2), (65, 4), (129, 4), (159, 4)]:
+        for L, slots in [(2, 2), (3, 2), (5, 2), (30, 2), (63, 2), (65, 4), (129, 4), (159, 4)]:  # (also rows shorter than a slot)
             p = _plan((1000, L))
             assert (p["family"], p["slots"], p["vec"], p["block"], p["workspace_bytes"]) == (F, slots, 4, 256, 0), (L, p)
             assert p["grid"] * 4 * 64 * slots * 4 >= 1000 * L
         assert _plan((1000, 121))["family"] == G and _plan((1000, 105))["family"] == F  # 28 to 32 lanes of a group: group
-        # not for whole slots, rows shorter than a slot or longer than 40, a single row, gaps, misaligned bases
-        for shape, kw in [((1000, 32), {}), ((1000, 3), {}), ((1000, 161), {}), ((1, 30), {}), ((1000, 30), dict(strides=(31, 1)))]:
+        # not for whole slots, rows of one element or longer than 40 slots, a single row, gaps, misaligned bases
+        for shape, kw in [((1000, 32), {}), ((1000, 1), {}), ((1000, 161), {}), ((1, 30), {}), ((1000, 30), dict(strides=(31, 1)))]:
             assert _plan(shape, **kw)["family"] != F, (shape, kw)
         assert nat.plan(torch.empty(30001)[1:].view(1000, 30))["family"] == nat.FAMILY_GROUP
         assert _plan((1000, 239), tuning=nat.Tuning(F))["family"] == F       # up to 60 slots on request
         with pytest.raises(NotImplementedError):
             _plan((1000, 241), tuning=nat.Tuning(F))
-        p = nat.plan(torch.empty(1000, 30, dtype=torch.bfloat16))
-        assert (p["family"], p["slots"], p["vec"]) == (F, 2, 8)
+        for L in (30, 4, 7):  # (16-bit storage: rows of half a slot as well)
+            p = nat.plan(torch.empty(1000, L, dtype=torch.bfloat16))
+            assert (p["family"], p["slots"], p["vec"]) == (F, 2, 8)
         assert nat.plan(torch.empty(1000, 32, dtype=torch.bfloat16))["family"] == nat.FAMILY_GROUP
         assert _plan((1000, 32), strides=(36, 1))["family"] == G      # padded rows that do
         p = _plan((1000, 5), strides=(8, 1))
