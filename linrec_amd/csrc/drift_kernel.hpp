@@ -40,10 +40,15 @@ namespace linrec {
 // one and two steps from now) and the tiles of loaded data change roles without a register being copied.
 // PF: tiles of loads in flight ahead of the scan (1 or 2); WPE: waves per SIMD the compiler is to allow for;
 // WIDE: teams of more than 64 are served (the forward with 16 waves of two slots has no registers for that).
-template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1, bool WIDE = true>
+// RAGGED: rows of whole slots whose last tile is a partial one (K = tiles of a row, the last one counted): that
+// tile takes the loads and stores that look at every slot, the others stay as they are; the team need not divide K,
+// and the walk's start moves on by K % M tiles in every row, so that neither the partial tiles nor the longer walks
+// all fall to the same team mates.
+template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int WPE = 1, bool WIDE = true, bool RAGGED = false>
 __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   static_assert(PF == 1 || PF == 2, "one or two tiles of loads ahead of the scan");
   static_assert(NW <= 16, "the waves' shares are composed inside a DPP row");
+  static_assert(!RAGGED || std::is_same_v<T, float>, "partial tiles: fp32 storage");
   constexpr int WAVE_SLOTS = S * 64;
   constexpr int TILE_SLOTS = NW * WAVE_SLOTS;
   __shared__ float sh_a[2][NW];
@@ -57,14 +62,22 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
 
   const int lane = threadIdx.x & 63;
   const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int M = p.tasks;          // team size, divides K
+  const int M = p.tasks;          // team size; divides K unless RAGGED
   const int K = p.tiles_per_row;  // every row is exactly K full tiles
   const int teams = int(p.row_groups);  // the grid is teams * M workgroups
   const int team = int(blockIdx.x) / M;
   const int j = int(blockIdx.x) - team * M;
   const int per_row = K / M;  // tiles of one row this walker takes: j, j + M, ...
   const long long my_rows = team < p.numseq ? (p.numseq - team + teams - 1) / teams : 0;
-  const int items = int(my_rows * per_row);
+  int items = int(my_rows * per_row);
+  const int rem = K - per_row * M;  // RAGGED: the team need not divide K
+  if constexpr (RAGGED) {
+    // A walk that starts at tile s < M takes one tile more than K / M where s < rem.  The starts of this walker's rows
+    // are j, j + rem, j + 2 rem, ... (mod M), which come to lie below rem once in every M / rem rows, evenly spaced (a
+    // walker that took the longer walk several rows running would fall behind its team mates by as many steps): as
+    // often as the sum passes a multiple of M.
+    if (my_rows > 0) items += (j < rem ? 1 : 0) + int((j + (my_rows - 1) * rem) / M);
+  }
 
   // (read through the scalar cache: it arrives beside the first tile's loads instead of holding them up, which an
   // agent-scope load did for a memory round trip at the start of every launch)
@@ -78,11 +91,17 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   };
   // the walk: tiles j, j + M, ... of row `team`, then of row team + teams, ...
   Item cursor = {team, j};
+  int turn = 0;  // RAGGED: how far the walk's start has moved on from j, K % M tiles a row
   auto next_item = [&]() {
     const Item it = cursor;
     cursor.t += M;
     if (cursor.t >= K) {
-      cursor.t = j;
+      if constexpr (RAGGED) {
+        turn = turn + rem >= M ? turn + rem - M : turn + rem;
+        cursor.t = j + turn >= M ? j + turn - M : j + turn;
+      } else {
+        cursor.t = j;
+      }
       cursor.row += teams;
     }
     return it;
@@ -274,14 +293,20 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
       tile_apply_store_packed<S, VEC, MODE, DESC>(q.d.ys, q.edge, q.r, ptrs_of(q.it.row), rv,
                                                   t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
     } else {
-      tile_apply_store<S, VEC, MODE, DESC, true>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS,
-                                                 lane, has_entry, entry);
+      if (RAGGED && t == K - 1)
+        tile_apply_store<S, VEC, MODE, DESC, false>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS,
+                                                    lane, has_entry, entry);
+      else
+        tile_apply_store<S, VEC, MODE, DESC, true>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS,
+                                                   lane, has_entry, entry);
     }
   };
   auto load_next = [&](Loaded& d, Item& it) {
     it = next_item();
     if constexpr (PACKED)
       tile_load_packed<S, VEC, MODE, DESC>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane);
+    else if (RAGGED && it.t == K - 1)
+      tile_load<S, VEC, MODE, DESC, false>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane, false);
     else
       tile_load<S, VEC, MODE, DESC, true>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane, false);
   };

@@ -72,6 +72,15 @@ KernelGroup kernels_bf16_cols();
   {PFX "drift_w" #NW "_s" #S "_" #MODE "_" #DESC,                                               \
    (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, VEC, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2 && (VEC) == 4)>, DT, LINREC_FAMILY_DRIFT, \
    NW, S, VEC, linrec::MODE, DESC, 1}
+// ... for rows of whole slots whose last tile is a partial one (`carry` column 2)
+#define DRIFT_RAGGED_ENTRY(TT, DT, PFX, NW, S, VEC, MODE, DESC)                                 \
+  {PFX "drift_ragged_w" #NW "_s" #S "_" #MODE "_" #DESC,                                        \
+   (const void*)&linrec::drift_kernel<TT, NW, S, VEC, linrec::MODE, DESC != 0, DRIFT_TILES_AHEAD(NW, S, VEC, MODE), ((NW) > 8 ? 4 : 2), !((NW) == 16 && (S) == 2 && (VEC) == 4), true>, DT, LINREC_FAMILY_DRIFT, \
+   NW, S, VEC, linrec::MODE, DESC, 2}
+#define DRIFT_RAGGED_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                         \
+  DRIFT_RAGGED_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_RAGGED_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
+#define DRIFT_RAGGED_BWD_DIRS(TT, DT, PFX, NW, S, VEC)                                         \
+  DRIFT_RAGGED_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 0), DRIFT_RAGGED_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_BWD, 1)
 #define DRIFT_FWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
   DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 0), DRIFT_ENTRY(TT, DT, PFX, NW, S, VEC, MODE_FWD, 1)
 #define DRIFT_BWD_DIRS(TT, DT, PFX, NW, S, VEC)                                                \
@@ -150,6 +159,8 @@ KernelGroup kernels_bf16_cols();
 #define SWEEP_(...) SWEEP_ALL_DIRS(__VA_ARGS__)
 #define DRIFT_FWD_(...) DRIFT_FWD_DIRS(__VA_ARGS__)
 #define DRIFT_BWD_(...) DRIFT_BWD_DIRS(__VA_ARGS__)
+#define DRIFT_RAGGED_FWD_(...) DRIFT_RAGGED_FWD_DIRS(__VA_ARGS__)
+#define DRIFT_RAGGED_BWD_(...) DRIFT_RAGGED_BWD_DIRS(__VA_ARGS__)
 #define TEAM_FWD_(...) TEAM_FWD_DIRS(__VA_ARGS__)
 #define STREAM_(...) STREAM_ALL_DIRS(__VA_ARGS__)
 #define COLUMN_(...) COLUMN_ALL_DIRS(__VA_ARGS__)

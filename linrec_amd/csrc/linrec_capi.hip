@@ -228,15 +228,24 @@ int64_t sweep_team_size(int64_t tiles_per_row, int64_t most = kSweepMaxTeam) {
 // teams only, every team the same number of rows where that is possible), the larger one of equals: the
 // more of a row is in flight at once, the fewer gaps the launch's reading positions leave.  A lane of a
 // wave per team mate: at most 64 a wave.
-int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int64_t resident) {
+int64_t drift_team_size(const Problem& q, int64_t tiles_per_row, int waves, int64_t resident, bool any_team = false,
+                        int64_t max_team = 0) {
   int64_t best = 1, best_large = 0;
   double best_busy = 0.0, best_large_busy = 0.0;
-  for (int64_t team = std::min<int64_t>({int64_t(64) * waves, resident, tiles_per_row}); team >= 1; --team) {
-    if (tiles_per_row % team != 0) continue;
+  if (max_team <= 0) max_team = int64_t(64) * waves;
+  for (int64_t team = std::min<int64_t>({max_team, resident, tiles_per_row}); team >= 1; --team) {
+    // (the kernels for rows with a partial last tile take teams that do not divide the tiles of a row)
+    if (tiles_per_row % team != 0 && !any_team) continue;
     const int64_t teams = std::min(q.numseq, resident / team);
     const int64_t rounds = ceil_div(q.numseq, teams);
-    const double busy = double(q.numseq * team) / double(rounds * resident);
-    if (busy > best_busy + 1e-9) {
+    // (a team that does not divide the tiles of a row: over the rows of a team some members take a tile more than others,
+    // and the members are never all in step - 1024 x 50000, seven tiles a row, in teams of 4 113.0 / 192.4 us, in teams
+    // of 7 108.0 / 174.9 us; 335 x 100000 backward, 25 tiles, in teams of 16 116.8 to 123.5 us, of 25 114.4 us)
+    const int64_t most = rounds * (tiles_per_row / team) + ceil_div(rounds * (tiles_per_row % team), team);
+    const double busy = double(q.numseq * team) / double(rounds * resident) *
+                        (double(rounds * tiles_per_row) / double(team * most)) * (tiles_per_row % team ? 0.93 : 1.0);
+    // (of such teams the larger one unless a smaller one keeps the chip 3 % busier: more of a row in flight at once)
+    if (busy > best_busy * (any_team && best_busy > 0.0 ? 1.03 : 1.0) + 1e-9) {
       best = team;
       best_busy = busy;
     }
@@ -321,13 +330,20 @@ int drift_slots_for(const Problem& q, int fv) {
       q.numseq * q.seqlen < kT_drift_bwd_few_rows_min_tiles_per_cu * 8192 * q.cus)
     return 0;
   if (little_work_in_many_rows(q)) return 0;
+  // Rows of whole tiles first; then rows of whole slots whose last tile is a partial one, in the forward's tiles of 8192
+  // elements and the backward's of 4096 (forward / backward in us against one workgroup per row or one team per row:
+  // 335 x 100000 69.8 / 114.6 against 83.4 / 142.9, 1024 x 50000 107.9 / 175.6 against 116.2 / 198.5, 100 x 250000
+  // 53.7 / 88.4 against 62.8 / 100.9, 512 x 60000 64.7 / 107.5 against 68.3 / 116.7).  The rules count their full tiles.
+  for (int pass = 0; pass < 2; ++pass)
   for (int s : {4, 2, 1}) {
+    const bool ragged = pass == 1;
     if (half != (s == 1)) continue;
     if (q.is_bwd && s == 4) continue;  // (the backward pass holds three tensors: two slots per lane fit)
     const int64_t tile = int64_t(8) * s * 64 * fv;
-    if (q.seqlen % tile != 0) continue;
-    const int64_t tiles_per_row = q.seqlen / tile;
-    const int64_t team = drift_team_size(q, tiles_per_row, 8, q.cus);
+    if ((q.seqlen % tile != 0) != ragged) continue;
+    if (ragged && (half || q.seqlen % fv != 0 || s != (q.is_bwd ? 2 : 4))) continue;
+    const int64_t tiles_per_row = q.seqlen / tile;  // (full ones)
+    const int64_t team = drift_team_size(q, tiles_per_row + ragged, 8, q.cus, ragged);
     // the forward's tiles of 8192 elements: as many tiles a row as the generated table says, and from its number of
     // rows on also rows of two tiles in teams of two (us, against one workgroup per row: 2048 x 16384 66.2 against 69.3,
     // 4096 x 16384 128.9 against 138.8; but 600 x 16384 22.6 against 22.1, 1024 x 16384 34.5 against 35.0)
@@ -335,7 +351,7 @@ int drift_slots_for(const Problem& q, int fv) {
                                 : q.numseq >= q.at(kT_drift_fwd_two_tiles_min_rows) ? 2 : kT_drift_fwd_min_tiles_per_row;
     if (tiles_per_row < least_tiles || team < least_tiles) continue;
     // (a caller that can only give so much workspace is served by the kernels that need less)
-    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
+    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * (tiles_per_row + ragged)) > q.workspace_cap) continue;
     // fp32 rows of fewer than eight tiles of 4096 elements: one workgroup per row does as well or better
     // (forward / backward in us: 768 x 16384 27.3 / 46.3 against 32.3 / 47.5, 400 x 24576 22.6 / 36.4 against
     // 26.3 / 39.7, 1000 x 24576 52.2 / 89.3 against 55.7 / 90.3, 1536 x 16384 52.4 / 90.4 against 55.3 / 89.7,
@@ -823,25 +839,27 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
     // 43.6, 1024 x 65536 132.2 against 133.8, 16 x 1048576 in teams of 128 37.6 against 38.1 - compiled without
     // the larger teams' code, which does not fit its registers, so those keep 8 waves).
     if (drift && !half && !q.is_bwd && auto_slots == 4 && !(tune && (tune->waves > 0 || tune->slots > 0)) &&
-        drift_team_size(q, q.seqlen / (int64_t(8) * 4 * 64 * fv), 8, q.cus) <= 64) {
+        drift_team_size(q, ceil_div(q.seqlen, int64_t(8) * 4 * 64 * fv), 8, q.cus, q.seqlen % (int64_t(8) * 4 * 64 * fv) != 0) <= 64) {
       waves = 16;
       slots = 2;
     }
     const int64_t tile_elems = int64_t(waves) * slots * 64 * fv;
-    // every tile of every row has to be a full one
-    if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || q.seqlen % tile_elems != 0) return LINREC_E_UNSUPPORTED;
-    const int id = find_kernel(q.dtype, family, waves, slots, fv, mode, desc, 1);
+    // every tile of every row has to be a full one; the drift kernels also come for rows of whole slots whose last
+    // tile is a partial one (kernel-table code 2 in the carry column)
+    const bool ragged = drift && q.seqlen % tile_elems != 0 && q.seqlen % fv == 0 && q.seqlen > tile_elems;
+    if (q.base_mis != 0 || (q.numseq > 1 && q.row_stride % fv != 0) || (q.seqlen % tile_elems != 0 && !ragged)) return LINREC_E_UNSUPPORTED;
+    const int id = find_kernel(q.dtype, family, waves, slots, fv, mode, desc, ragged ? 2 : 1);
     if (id < 0) return LINREC_E_UNSUPPORTED;
     const int block = 64 * waves;
-    const int64_t tiles_per_row = q.seqlen / tile_elems;
+    const int64_t tiles_per_row = ceil_div(q.seqlen, tile_elems);
     // Every workgroup of the launch has to be resident at once (a walker waits for its team mates, and a
     // workgroup that has not started yet only starts when another one ends): never more than the CUs hold.
     const int64_t resident = int64_t(workgroups_per_cu(id, block, drift || q.is_bwd ? 1 : 2)) * q.cus;
     const int64_t team = tune && tune->tasks > 0
                              ? tune->tasks
-                             : drift ? drift_team_size(q, tiles_per_row, waves, resident)
+                             : drift ? drift_team_size(q, tiles_per_row, waves, resident, ragged, ragged ? drift_max_team(waves, slots, fv) : 0)
                                      : sweep_team_size(tiles_per_row, std::min<int64_t>(kSweepMaxTeam, resident));
-    if (team > (drift ? drift_max_team(waves, slots, fv) : 64) || team > tiles_per_row || tiles_per_row % team != 0) return LINREC_E_UNSUPPORTED;
+    if (team > (drift ? drift_max_team(waves, slots, fv) : 64) || team > tiles_per_row || (tiles_per_row % team != 0 && !ragged)) return LINREC_E_UNSUPPORTED;
     int64_t teams = tune && tune->carry > 0 ? tune->carry : std::min(sweep_workgroups(q), resident) / team;
     if (teams > q.numseq) teams = q.numseq;
     if (teams < 1 || teams * team > resident) return LINREC_E_UNSUPPORTED;

@@ -297,12 +297,12 @@ _DRIFT = {"fwd": _t(nat.FAMILY_DRIFT, 16, 2), "bwd": _t(nat.FAMILY_DRIFT, 16, 1)
 _DRIFT_SMALL = {"fwd": _t(nat.FAMILY_DRIFT, 16, 1), "bwd": _t(nat.FAMILY_DRIFT, 16, 1)}
 
 CROSSOVERS = [
-    Crossover("stream_min_rows", "ragged long rows (65540 elements): one team of workgroups per row against one "
-              "workgroup per row, by the number of rows", [64, 96, 112, 128, 129, 144, 160, 192],
-              lambda v: (v, 65540), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_STREAM))),
-    Crossover("team_min_rows", "a few ragged very long rows (1048580 elements): look-back tiles against one team of "
-              "64 workgroups per row, by the number of rows", [2, 3, 4, 5, 6, 8, 12],
-              lambda v: (v, 1048580), _both(_t(nat.FAMILY_TILE, 8, 8, 1, 1)), _both(_t(nat.FAMILY_TEAM))),
+    Crossover("stream_min_rows", "long rows that are not whole slots (65542 elements): one team of workgroups per row "
+              "against one workgroup per row, by the number of rows", [64, 96, 112, 128, 129, 144, 160, 192],
+              lambda v: (v, 65542), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_STREAM))),
+    Crossover("team_min_rows", "a few very long rows that are not whole slots (1048582 elements): look-back tiles against "
+              "one team of 64 workgroups per row, by the number of rows", [2, 3, 4, 5, 6, 8, 12],
+              lambda v: (v, 1048582), _both(_t(nat.FAMILY_TILE, 8, 8, 1, 1)), _both(_t(nat.FAMILY_TEAM))),
     Crossover("drift_bwd_max_rows", "backward of many rows of 32768 elements: drift teams (tiles stored two steps "
               "late) against sweep teams (tiles of 8192 elements, exchange waited for), by the number of rows",
               [1024, 1536, 2048, 3072, 4096], lambda v: (v, 32768), _DRIFT_SMALL, _both(_t(nat.FAMILY_SWEEP, 8, 4)),

@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 
 CASES = {
     # name: (numseq, seqlen, transposed, reverse, dtype, expected family)
-    "stream_f32": (70144, 32776, False, False, torch.float32, "STREAM"),
+    "stream_f32": (70144, 32778, False, False, torch.float32, "STREAM"),       # rows that are not whole slots
+    "drift_ragged_f32": (70144, 32776, False, False, torch.float32, "DRIFT"),  # whole slots, a partial last tile
     "drift_rows_f32": (56000, 40960, False, False, torch.float32, "DRIFT"),  # (its backward: teams that wait, SWEEP)
     "tile_f32": (1100000, 2048, False, True, torch.float32, "TILE"),
     "flat_f32": (72000000, 30, False, True, torch.float32, "FLAT"),
@@ -22,7 +23,7 @@ CASES = {
     "coldrift_f32": (4000, 537000, True, True, torch.float32, "COLDRIFT"),
     "colblock_f32": (16000, 134300, True, True, torch.float32, "COLUMN"),
     "drift_f32": (20, 1 << 27, False, True, torch.float32, "DRIFT"),  # (its backward: teams that wait, SWEEP)
-    "team_f32": (18, (1 << 27) + 12, False, False, torch.float32, "TEAM"),
+    "team_f32": (18, (1 << 27) + 14, False, False, torch.float32, "TEAM"),
     "stream_bf16": (70000, 32768, False, True, torch.bfloat16, "STREAM"),
 }
 

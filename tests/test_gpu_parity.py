@@ -46,15 +46,28 @@ def _run_both(nat, x, c, dy, reverse, tuning, label):
     assert nat.gave_up_count() == 0
 
 
-def _run_forward(nat, x, c, reverse, tuning, label):
-    """The forward pass alone (geometries that are compiled for the forward only)."""
+def _run_forward(nat, x, c, reverse, tuning, label, check_gave_up=True):
+    """The forward pass alone (geometries that are compiled for the forward only); returns the device's outputs."""
     y_t = truth(x, c, torch.zeros_like(x), reverse)[0]
     dev = torch.device("cuda:0")
     xd, cd = x.to(dev), c.to(dev)
     y = nat.fwd(xd, cd, reverse, tuning, out=_nan_like(xd))
     torch.cuda.synchronize()
     check_close(y, y_t, f"{label} outputs")
-    assert nat.gave_up_count() == 0
+    assert not check_gave_up or nat.gave_up_count() == 0
+    return y
+
+
+def _run_backward(nat, dy, c, y, reverse, tuning, label, check_gave_up=True):
+    """The backward pass alone, from outputs `y` that a forward left on the device."""
+    dev = torch.device("cuda:0")
+    dx_t, dc_t = oracle.bwd(dy.numpy().astype(np.float64), c.numpy().astype(np.float64),
+                            y.cpu().numpy().astype(np.float64), reverse, dtype=np.float64)
+    dx, dc = nat.bwd(dy.to(dev), c.to(dev), y, reverse, tuning, out=(_nan_like(y), _nan_like(y)))
+    torch.cuda.synchronize()
+    check_close(dx, dx_t, f"{label} d_inputs")
+    check_close(dc, dc_t, f"{label} d_coeffs")
+    assert not check_gave_up or nat.gave_up_count() == 0
 
 
 def _tunings_for(nat, L):
@@ -858,6 +871,61 @@ def test_drift_teams_of_more_than_one_collecting_wave(nat, rows, tiles, slots, t
         _run_both(nat, x, c, dy, reverse, tuning, label)
     else:
         _run_forward(nat, x, c, reverse, tuning, label)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_rows_with_a_partial_last_tile_run_in_drift_teams(nat, reverse):
+    """fp32 rows of whole 16-byte slots whose length is not a whole number of tiles: the drift kernels' last tile of a
+    row is a partial one (down to a single slot, up to a tile less a slot), the teams need not divide the tiles of a
+    row, and the walk starts one tile further along in every row.  Forced geometries and team sizes on few and many
+    rows, the planner's own choice, and a poll limit of one."""
+    D = nat.FAMILY_DRIFT
+    dev = torch.device("cuda:0")
+    names = nat.kernel_table()
+    for shape, teams in [((3, 8192 * 2 + 4), (0, 2, 3)), ((5, 8192 * 3 + 4096), (0, 3)), ((7, 8192 * 5 - 4), (0, 4, 5)),
+                         ((33, 8192 * 4 + 1000), (0, 2, 5)), ((260, 8192 * 2 + 8), (0,)), ((2, 8192 * 13 + 8188), (0, 9, 14)),
+                         ((1, 8192 * 40 + 12), (0, 7, 41))]:
+        x, c, dy = make_inputs(shape, "near1", seed=shape[0] * 1000 + shape[1] % 977)
+        for team in teams:
+            for fw, bw in [((16, 2), (16, 1)), ((8, 4), (16, 1))]:
+                tf = nat.Tuning(D, fw[0], fw[1], -1, team)
+                # (the backward's tiles are half the forward's: twice the team, where one is asked for; rows of whole
+                # such tiles take the kernel for them, whose teams divide the tiles of a row)
+                kb = -(-shape[1] // 4096)
+                team_b = min(2 * team, kb)
+                if team_b and shape[1] % 4096 == 0 and kb % team_b:
+                    team_b = kb
+                tb = nat.Tuning(D, bw[0], bw[1], -1, team_b)
+                pf, pb = nat.plan(x.to(dev), reverse, False, tf), nat.plan(x.to(dev), reverse, True, tb)
+                assert "ragged" in names[pf["kernel_id"]] and pf["tiles_per_row"] == -(-shape[1] // 8192), pf
+                assert ("ragged" in names[pb["kernel_id"]]) == (shape[1] % 4096 != 0) and pb["tiles_per_row"] == -(-shape[1] // 4096), pb
+                if team:
+                    assert pf["tasks"] == team, pf
+                label = f"drift {shape} forward {fw} team {pf['tasks']}, backward team {pb['tasks']}"
+                y = _run_forward(nat, x, c, reverse, tf, label)
+                _run_backward(nat, dy, c, y, reverse, tb, label)
+    assert nat.gave_up_count() == 0
+    # the planner's own choice: teams that fill the chip, whatever the tiles of a row
+    for shape, fwd, bwd in [((335, 100000), (16, 2, 13), (16, 1, 25)), ((100, 250000), (16, 2, 28), (16, 1, 61)),
+                            ((16, 1000000), (8, 4, 123), (16, 1, 245)), ((1024, 50000), (16, 2, 7), (16, 1, 13))]:
+        x, c, dy = make_inputs(shape, "sigmoid", seed=shape[0])
+        for is_bwd, want in ((False, fwd), (True, bwd)):
+            plan = nat.plan(x.to(dev), reverse, is_bwd)
+            assert plan["family"] == D and "ragged" in names[plan["kernel_id"]], plan
+            assert (plan["waves"], plan["slots"]) == want[:2] and plan["grid"] <= 256 and plan["grid"] % plan["tasks"] == 0, plan
+        _run_both(nat, x, c, dy, reverse, None, f"drift {shape}, default plan")
+    assert nat.gave_up_count() == 0
+    # a poll limit of one: waits run out, the value entering a tile comes from the row's own data instead
+    x, c, dy = make_inputs((6, 8192 * 50 + 5000), "near1", seed=4)
+    old = nat.lib().linrec_set_spin_limit(1)
+    try:
+        y = _run_forward(nat, x, c, reverse, nat.Tuning(D, 16, 2, -1, 17), "poll limit 1, forward", check_gave_up=False)
+        _run_backward(nat, dy, c, y, reverse, nat.Tuning(D, 16, 1, -1, 33), "poll limit 1, backward", check_gave_up=False)
+    finally:
+        nat.lib().linrec_set_spin_limit(old)
+    print("drift with partial tiles, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
+    for ws in list(nat._workspaces.values()):
+        ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
 
 
 @pytest.mark.parametrize("kind", ["look-back", "chain", "team", "sweep", "drift", "drift-200", "drift-16-waves"])

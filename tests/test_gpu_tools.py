@@ -15,7 +15,7 @@ def test_tuning_sweep_checks_every_geometry_against_the_sequential_path():
     def worst(r):  # a pass a geometry is not compiled for reports nan
         return max(d for d in (r["fwd_err_vs_sequential"], r["bwd_err_vs_sequential"]) if d == d)
 
-    rows = tune.sweep((96, 20000), iters=3, warmup=1, sets=1)
+    rows = tune.sweep((96, 20002), iters=3, warmup=1, sets=1)  # (rows that are not whole slots: no drift kernels)
     assert len(rows) > 10
     kinds = {r["geometry"].split()[0] for r in rows}
     assert {"table", "tile", "chain", "stream"} <= kinds

@@ -98,7 +98,7 @@ def test_planner_follows_the_compute_unit_count():
                 assert p["grid"] <= cus and p["grid"] % p["tasks"] == 0
                 seen[(cus, is_bwd)] = p["grid"]
             # one team of workgroups per row: never more workgroups than CUs
-            t = nat.plan(torch.empty(8, 1048580), False, False)
+            t = nat.plan(torch.empty(8, 1048579), False, False)  # (rows that are not whole slots)
             assert t["family"] == nat.FAMILY_TEAM and t["grid"] <= cus and t["tasks"] == cus // 8
             # a single very long row: one team of the whole device
             w = nat.plan(torch.empty(1, 1 << 25), False, False)
@@ -110,8 +110,8 @@ def test_planner_follows_the_compute_unit_count():
                 if c["family"] == nat.FAMILY_COLDRIFT:
                     assert c["grid"] == 64 * c["tasks"] <= cus
             # one workgroup per row from half the CUs on, teams below
-            assert nat.plan(torch.empty(cus // 2 + 1, 65540))["family"] == nat.FAMILY_STREAM
-            assert nat.plan(torch.empty(cus // 2, 65540))["family"] == nat.FAMILY_TEAM
+            assert nat.plan(torch.empty(cus // 2 + 1, 65542))["family"] == nat.FAMILY_STREAM
+            assert nat.plan(torch.empty(cus // 2, 65542))["family"] == nat.FAMILY_TEAM
         assert seen[(256, False)] == 256 and seen[(128, False)] == 128 and seen[(64, False)] == 64
         assert seen[(256, True)] == 256 and seen[(128, True)] == 128 and seen[(64, True)] == 64
         # a team that cannot be resident at once is refused rather than left to wait for absent mates
@@ -217,7 +217,10 @@ class TestPlanner:
         assert (p4["tasks"], p4["grid"], p4["tiles_per_row"]) == (128, 256, 128)
         p4bw = _plan((16, 1048576), is_bwd=True)  # the backward: one team of the whole launch, tiles of 4096 elements
         assert (p4bw["family"], p4bw["waves"], p4bw["slots"], p4bw["tasks"], p4bw["grid"], p4bw["tiles_per_row"]) == (nat.FAMILY_DRIFT, 16, 1, 256, 256, 256)
-        p4r = _plan((16, 1048576 + 4))  # a ragged last tile: one team per row
+        p4d = _plan((16, 1048576 + 4))  # whole slots, a partial last tile: the drift kernels all the same
+        assert p4d["family"] == nat.FAMILY_DRIFT and p4d["tiles_per_row"] == 129 and "drift_ragged_w8_s4" in names[p4d["kernel_id"]]
+        assert p4d["tasks"] == 128 and p4d["grid"] == 256  # (a team need not divide the tiles of such a row)
+        p4r = _plan((16, 1048576 + 3))  # rows that are not whole slots: one team per row
         assert p4r["family"] == nat.FAMILY_TEAM and p4r["grid"] == 16 * p4r["tasks"] and 2 <= p4r["tasks"] <= 64
         for rows, is_bwd in ((1, False), (2, False), (3, True), (6, True)):
             # a few very long rows: one team of the whole chip, every wave of a workgroup collecting maps
@@ -321,7 +324,7 @@ class TestPlanner:
         assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 2, 8, 256), q
         m = T["drift_bwd_max_rows"]
         assert 1024 <= m and fam((m, 65536), True) == D and fam((m + 256, 65536), True) == W
-        assert fam((m + 256, 131072), True) == ST and fam((4096, 65536 + 8)) == ST
+        assert fam((m + 256, 131072), True) == ST and fam((4096, 65536 + 6)) == ST and fam((4096, 65536 + 8)) == D
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
         # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
@@ -329,16 +332,17 @@ class TestPlanner:
         assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
-        assert slots((700, 24576)) == 4 and slots((838, 40000)) == 4 and slots((800, 36000)) == 2
-        assert fam((300, 65536 + 4)) == nat.FAMILY_STREAM          # ragged last tile
+        assert slots((700, 24576)) == 4 and slots((838, 40002)) == 4 and slots((800, 36002)) == 2
+        assert fam((300, 65536 + 6)) == nat.FAMILY_STREAM          # rows that are not whole slots
+        assert fam((300, 65536 + 4)) == D and fam((838, 40000)) == D   # whole slots, a partial last tile: drift teams
         # ... whose rows beyond one per CU, if few, go to a second launch of their own (teams per row)
-        p = nat.plan(torch.empty(300, 65536 + 4))
+        p = nat.plan(torch.empty(300, 65536 + 6))
         assert (p["tail_rows"], p["grid"]) == (44, 256) and p["workspace_bytes"] > 0
-        assert [nat.plan(torch.empty(n, 65536 + 4))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
-        assert nat.plan(torch.empty(300, 65536 + 4), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
+        assert [nat.plan(torch.empty(n, 65536 + 6))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
+        assert nat.plan(torch.empty(300, 65536 + 6), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
         assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
-        assert fam((T["team_min_rows"], (1 << 20) + 4)) == nat.FAMILY_TEAM          # few ragged rows: one team per row
-        assert fam((T["team_min_rows"] - 1, (1 << 20) + 4)) == nat.FAMILY_TILE      # fewer: look-back tiles
+        assert fam((T["team_min_rows"], (1 << 20) + 6)) == nat.FAMILY_TEAM          # few rows that are not whole slots: one team per row
+        assert fam((T["team_min_rows"] - 1, (1 << 20) + 6)) == nat.FAMILY_TILE      # fewer: look-back tiles
         assert fam((300, 65536 + 8), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
         # 16-bit storage: teams whose tiles are stored two steps late serve the backward of up to drift_bwd_max_rows
         # rows of whole tiles of 8192 elements (16 waves of one slot) and the forward of any number of rows of four and
@@ -600,7 +604,7 @@ class TestPlanner:
         assert lib.linrec_plan_f32(None, 4, 10, 5, 1, 0, 0, None, ctypes.byref(plan)) == -1  # rows overlap
         assert lib.linrec_plan_f32(None, 4, 2 ** 31, 2 ** 31, 1, 0, 0, None, ctypes.byref(plan)) == -4
         assert lib.linrec_workspace_bytes(16, 1 << 20, 1 << 20, 1, 0, 0, None) > 0
-        assert lib.linrec_workspace_bytes(4096, 65540, 65540, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
+        assert lib.linrec_workspace_bytes(4096, 65542, 65542, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
         assert lib.linrec_workspace_bytes_for_tiles(0) == 0
         assert lib.linrec_workspace_bytes_for_tiles(1000) >= 16 + 16 * 1000
 
