@@ -73,7 +73,10 @@ extern "C" {
                                   fp32 forward 8 x 4, 8 x 2, 4 x 4, 16 x 1 and 16 x 2 (the last for teams of at most
                                   64 only), fp32 backward 8 x 2 and 16 x 1; 16-bit storage (slots of eight
                                   elements) forward 16 x 2, 16 x 1 and 8 x 1, backward 16 x 1.
-                                  The planner's picks are the 16-wave ones, and 8 x 4 forward for fp32 teams beyond 64 */
+                                  The planner's picks are the 16-wave ones, and 8 x 4 forward for fp32 teams beyond 64.
+                                  Rows must be whole tiles; fp32 rows of whole 16-byte slots may end in a partial
+                                  tile (forward 16 x 2 and 8 x 4, backward 16 x 1), and their teams need not divide
+                                  the tiles of a row */
 
 #define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
                                    of workgroups share a block of rows and take its steps along the scan axis in
