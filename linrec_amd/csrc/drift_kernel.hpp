@@ -48,7 +48,6 @@ template <typename T, int NW, int S, int VEC, int MODE, bool DESC, int PF, int W
 __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   static_assert(PF == 1 || PF == 2, "one or two tiles of loads ahead of the scan");
   static_assert(NW <= 16, "the waves' shares are composed inside a DPP row");
-  static_assert(!RAGGED || std::is_same_v<T, float>, "partial tiles: fp32 storage");
   constexpr int WAVE_SLOTS = S * 64;
   constexpr int TILE_SLOTS = NW * WAVE_SLOTS;
   __shared__ float sh_a[2][NW];
@@ -284,14 +283,14 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
         k.xs[j] = from[(2 * j) * 64];
         k.cs[j] = from[(2 * j + 1) * 64];
       }
-      tile_replay_store_packed<S, VEC, DESC>(k, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
-                                             t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+      tile_replay_store_packed<S, VEC, DESC, RAGGED>(k, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
+                                                     t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
     } else if constexpr (REPLAY) {
-      tile_replay_store_packed<S, VEC, DESC>(q.d, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
-                                             t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+      tile_replay_store_packed<S, VEC, DESC, RAGGED>(q.d, q.r, t == 0 && wave == 0 && lane == 0, ptrs_of(q.it.row), rv,
+                                                     t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
     } else if constexpr (PACKED) {
-      tile_apply_store_packed<S, VEC, MODE, DESC>(q.d.ys, q.edge, q.r, ptrs_of(q.it.row), rv,
-                                                  t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
+      tile_apply_store_packed<S, VEC, MODE, DESC, RAGGED>(q.d.ys, q.edge, q.r, ptrs_of(q.it.row), rv,
+                                                          t * TILE_SLOTS + wave * WAVE_SLOTS, lane, has_entry, entry);
     } else {
       if (RAGGED && t == K - 1)
         tile_apply_store<S, VEC, MODE, DESC, false>(q.d, q.r, ptrs_of(q.it.row), rv, t * TILE_SLOTS + wave * WAVE_SLOTS,
@@ -303,8 +302,8 @@ __global__ __launch_bounds__(64 * NW, WPE) void drift_kernel(TileArgs p) {
   };
   auto load_next = [&](Loaded& d, Item& it) {
     it = next_item();
-    if constexpr (PACKED)
-      tile_load_packed<S, VEC, MODE, DESC>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane);
+    if constexpr (PACKED)  // (16-bit storage: a slot either lies in the row or beyond its end, every tile asks)
+      tile_load_packed<S, VEC, MODE, DESC, RAGGED>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane);
     else if (RAGGED && it.t == K - 1)
       tile_load<S, VEC, MODE, DESC, false>(d, ptrs_of(it.row), rv, it.t * TILE_SLOTS + wave * WAVE_SLOTS, lane, false);
     else

@@ -180,7 +180,8 @@ KernelGroup kernels_bf16_cols();
   TILE_(TY, 8, 2, 8, 0), TILE_(TY, 16, 2, 8, 0), TILE_(TY, 4, 2, 8, 1), TILE_(TY, 8, 4, 8, 1),  \
   TILE_(TY, 4, 4, 1, 0), TILE_(TY, 4, 4, 1, 1), STREAM_(TY, 8, 2, 8), TEAM_(TY, 8, 2, 8),       \
   TEAM_FWD_(TY, 8, 4, 8), SWEEP_(TY, 8, 2, 8), DRIFT_FWD_(TY, 8, 1, 8),                            \
-  DRIFT_FWD_(TY, 16, 1, 8), DRIFT_BWD_(TY, 16, 1, 8), DRIFT_FWD_(TY, 16, 2, 8)
+  DRIFT_FWD_(TY, 16, 1, 8), DRIFT_BWD_(TY, 16, 1, 8), DRIFT_FWD_(TY, 16, 2, 8),                     \
+  DRIFT_RAGGED_FWD_(TY, 16, 2, 8), DRIFT_RAGGED_BWD_(TY, 8, 2, 8)
 #define HALF_COLUMN_KERNELS(TY)                                                                 \
   GROUP_(TY, 8), FLAT_(TY, 8, 2),                                                               \
   COLUMN_(TY, 8, 4), COLUMN_(TY, 4, 8), COLUMN_(TY, 2, 8), COLUMN_(TY, 2, 16), COLUMN_(TY, 1, 8), COLUMN_(TY, 1, 16), \

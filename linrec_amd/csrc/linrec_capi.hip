@@ -287,18 +287,24 @@ int64_t drift_max_team(int waves, int slots, int vec) { return waves == 16 && sl
 // 1 x 33554432 38.6 against 42.9, 64 x 524288 37.0 against 39.6, 300 x 65536 24.0 against 25.6 / 26.9 for one workgroup
 // per row, 1024 x 131072 136.6 against 145.9 / 141.4, 512 x 65536 36.7 against 38.6 / 37.3; rows of two tiles:
 // 2048 x 32768 70.9 against 67.9).
+// Rows of whole slots whose last tile is a partial one (second pass, as for fp32): the forward's tiles of 16384
+// elements, the backward's of 8192 in 8 waves of two slots (16 waves of one have no registers left for the slots that
+// lie beyond the row's end); the rules count the full tiles.
 int half_drift_slots_for(const Problem& q, int fv) {
   if (q.is_bwd && q.numseq > q.at(kT_drift_bwd_max_rows)) return 0;
+  for (int pass = 0; pass < 2; ++pass)
   for (int s : {4, 2, 1}) {
+    const bool ragged = pass == 1;
     if (s == 4 && q.is_bwd) continue;
     if (s == 1 && (q.is_bwd || q.numseq > 2)) continue;
     const int64_t tile = int64_t(8) * s * 64 * fv;
-    if (q.seqlen % tile != 0) continue;
-    const int64_t tiles_per_row = q.seqlen / tile;
+    if ((q.seqlen % tile != 0) != ragged) continue;
+    if (ragged && (q.seqlen % fv != 0 || s != (q.is_bwd ? 2 : 4))) continue;
+    const int64_t tiles_per_row = q.seqlen / tile;  // (full ones)
     if (s != 4 && !q.is_bwd && q.numseq > q.at(kT_half_drift_fwd_small_tiles_max_rows) && !(q.numseq < q.at(256) && tiles_per_row >= 32)) continue;
-    const int64_t team = drift_team_size(q, tiles_per_row, s == 1 ? 8 : 16, q.cus);
+    const int64_t team = drift_team_size(q, tiles_per_row + ragged, s == 1 ? 8 : 16, q.cus, ragged);
     if (tiles_per_row < kSweepMinTiles || team < kSweepMinTiles) continue;
-    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * tiles_per_row) > q.workspace_cap) continue;
+    if (q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * (tiles_per_row + ragged)) > q.workspace_cap) continue;
     // the teams have to fill at least half the chip, and every member gets a few tiles: the backward and a few rows'
     // forward (fewer than a quarter of the compute units) as many for each compute unit as the generated table says
     // (the forward's in tiles of 16384 elements, so twice as many of 8192), more rows forward four of them (200 x 65536
@@ -820,6 +826,11 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
         (auto_slots == 2 || (auto_slots == 0 && q.seqlen % (int64_t(16) * 64 * fv) == 0))) {
       waves = 16;
       slots = 1;
+      // (the backward of rows with a partial last tile: 8 waves of two slots)
+      if (q.is_bwd && q.seqlen % (int64_t(16) * 64 * fv) != 0) {
+        waves = 8;
+        slots = 2;
+      }
     }
     // ... and its forward tiles of 16384 elements: 16 waves with two slots each
     if (drift && half && auto_slots == 4 && !(tune && (tune->waves > 0 || tune->slots > 0))) {

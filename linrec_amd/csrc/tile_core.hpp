@@ -187,30 +187,43 @@ struct TilePacked {
 };
 
 // The loads of tile_load<..., INTERIOR = true>, in the same order, without the conversion.
-template <int S, int VEC, int MODE, bool DESC, typename T>
+// MASKED: the row is whole slots (rv.lo == 0, its length a multiple of VEC) and ends inside this tile: a slot lies in
+// the row or beyond its end, and the slots beyond it read as inputs of zero and coefficients of one.
+template <int S, int VEC, int MODE, bool DESC, bool MASKED = false, typename T>
 __device__ __forceinline__ void tile_load_packed(TilePacked<T, S, VEC, MODE>& d, const RowPtrs<T>& q, const RowView& rv,
                                                  int u_wave, int lane) {
   static_assert(VEC > 1, "whole slots");
   using V = typename Pack<T, VEC>::type;
+  // (with MASKED this may lie in front of the row: only slots of the row are read)
   const long long s_low = DESC ? (long long)rv.nslots - u_wave - S * 64 : (long long)u_wave;
   const V* bx = reinterpret_cast<const V*>(q.in0) + s_low;
   const V* bc = reinterpret_cast<const V*>(q.coef) + s_low;
   const V* by = MODE == MODE_BWD ? reinterpret_cast<const V*>(q.aux) + s_low : nullptr;
   const unsigned lane_idx = DESC ? 63u - unsigned(lane) : unsigned(lane);
+  // (a slot beyond the row: the registers are set first and the load is skipped)
+  auto load_or = [&](V& to, const V* from, int j, float fill) {
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) to[i] = T(fill);
+      if (u_wave + j * 64 + lane < rv.nslots) to = stream_load(from);
+    } else {
+      to = stream_load(from);
+    }
+  };
 #pragma unroll
   for (int j = 0; j < S; ++j) {
-    d.xs[j] = stream_load(bx + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    load_or(d.xs[j], bx + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx, j, 0.0f);
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
   for (int j = 0; j < S; ++j) {
-    d.cs[j] = stream_load(bc + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    load_or(d.cs[j], bc + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx, j, 1.0f);
     __builtin_amdgcn_sched_barrier(0);
   }
   if constexpr (MODE == MODE_BWD) {
 #pragma unroll
     for (int j = 0; j < S; ++j) {
-      d.ys[j] = stream_load(by + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+      load_or(d.ys[j], by + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx, j, 0.0f);
       __builtin_amdgcn_sched_barrier(0);
     }
     d.y_edge = T(0.0f);
@@ -464,7 +477,7 @@ __device__ __forceinline__ void tile_scan_packed_fwd(const TilePacked<T, S, VEC,
 
 // ... and the second scan: every lane runs the recurrence over its slots' elements from the value that enters the
 // slot, rounds and packs the results as they come, and the stores go out back to back.
-template <int S, int VEC, bool DESC, typename T>
+template <int S, int VEC, bool DESC, bool MASKED = false, typename T>
 __device__ __forceinline__ void tile_replay_store_packed(const TilePacked<T, S, VEC, MODE_FWD>& k, const TileScan<S, VEC>& r,
                                                          bool row_first_lane, const RowPtrs<T>& q, const RowView& rv,
                                                          int u_wave, int lane, bool has_entry, float entry) {
@@ -487,7 +500,8 @@ __device__ __forceinline__ void tile_replay_store_packed(const TilePacked<T, S, 
   }
 #pragma unroll
   for (int j = 0; j < S; ++j) {
-    stream_store(o[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    if (!MASKED || u_wave + j * 64 + lane < rv.nslots)  // (MASKED: rows of whole slots that end inside this tile)
+      stream_store(o[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -497,7 +511,7 @@ __device__ __forceinline__ void tile_replay_store_packed(const TilePacked<T, S, 
 // not S * VEC floats.  The caller has folded each slot's map from the wave's entry value into the elements' maps
 // (ex_a = 1, ex_b = 0, and pa[j][0] is a factor like the others, also in the backward).  `y_edge`: the saved output
 // after the wave's last (what lane 63 needs; wave-uniform).
-template <int S, int VEC, int MODE, bool DESC, typename T>
+template <int S, int VEC, int MODE, bool DESC, bool MASKED = false, typename T>
 __device__ __forceinline__ void tile_apply_store_packed(const typename Pack<T, VEC>::type* ys, float y_edge,
                                                         const TileScan<S, VEC>& r, const RowPtrs<T>& q, const RowView& rv,
                                                         int u_wave, int lane, bool has_entry, float entry) {
@@ -529,13 +543,15 @@ __device__ __forceinline__ void tile_apply_store_packed(const typename Pack<T, V
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int j = 0; j < S; ++j) {
-    stream_store(o0[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+    if (!MASKED || u_wave + j * 64 + lane < rv.nslots)  // (MASKED: rows of whole slots that end inside this tile)
+      stream_store(o0[j], b0 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
     __builtin_amdgcn_sched_barrier(0);
   }
   if constexpr (MODE == MODE_BWD) {
 #pragma unroll
     for (int j = 0; j < S; ++j) {
-      stream_store(o1[j], b1 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
+      if (!MASKED || u_wave + j * 64 + lane < rv.nslots)
+        stream_store(o1[j], b1 + (DESC ? unsigned(S - 1 - j) : unsigned(j)) * 64u + lane_idx);
       __builtin_amdgcn_sched_barrier(0);
     }
   }

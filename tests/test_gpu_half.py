@@ -198,14 +198,15 @@ def test_config_shapes_through_autograd(name, shape, coeffs, reverse, transposed
 @pytest.mark.parametrize("reverse", [False, True])
 def test_a_few_very_long_rows(nat, reverse, dtype):
     """One or two very long rows run in teams that fill the launch (four and two collecting waves), both passes where
-    the rows are whole tiles of 8192 elements and the forward alone where they are whole tiles of 4096 only; three to
+    the rows are whole tiles of 8192 elements; where they are whole tiles of 4096 only, the forward in those and the
+    backward in tiles of 8192 of which the last is half full; three to
     five rows with less than four tiles for every compute unit, or ragged ones, run forward in teams of up to 64 and
     backward in look-back tiles.  Also with a poll limit of one: every wait of the team members for each other's maps
     may run out, and the results are the same."""
     dev = torch.device("cuda:0")
     D, TM, TL = nat.FAMILY_DRIFT, nat.FAMILY_TEAM, nat.FAMILY_TILE
     for shape, fwd, bwd in [((1, 8192 * 512), (D, 16, 1, 256), (D, 16, 1, 256)), ((2, 8192 * 300), (D, 16, 1, 100), (D, 16, 1, 100)),
-                            ((2, 4096 * 605), (D, 8, 1, 121), (TL, 8, 4, 1)),
+                            ((2, 4096 * 605), (D, 8, 1, 121), (D, 8, 2, 101)),
                             ((4, 16384 * 512), (D, 16, 2, 256), (D, 16, 1, 256)), ((5, 16384 * 231), (D, 16, 2, 231), (D, 16, 1, 231)),
                             ((3, 4096 * 300), (TM, 8, 4, 64), (TL, 8, 4, 1)), ((5, 4096 * 150 + 24), (TM, 8, 4, 38), (TL, 8, 4, 1))]:
         x, c, dy = _inputs(shape, dtype, seed=shape[0], coeffs="near1")
@@ -305,6 +306,70 @@ def test_column_drift_kernels_two_rows_per_lane(nat, reverse, dtype):
     finally:
         nat.lib().linrec_set_spin_limit(old)
     print("16-bit column drift, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
+    for ws in list(nat._workspaces.values()):
+        ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
+    _check(y, oracle.fwd(f64(x), f64(c), reverse), dtype, "poll limit 1 outputs")
+    dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y_kept.cpu()), reverse)
+    _check(dx, dx_t, dtype, "poll limit 1 d_inputs")
+    _check(dc, dc_t, dtype, "poll limit 1 d_coeffs")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_rows_with_a_partial_last_tile_run_in_drift_teams(nat, reverse, dtype):
+    """16-bit rows of whole slots of eight elements whose length is not a whole number of tiles: the drift kernels'
+    last tile of a row is a partial one (every slot lies in the row or beyond its end), the teams need not divide the
+    tiles of a row.  The forward in tiles of 16384 elements, the backward in tiles of 8192 in 8 waves of two slots.
+    Forced team sizes, the planner's own choice, and a poll limit of one."""
+    D = nat.FAMILY_DRIFT
+    dev = torch.device("cuda:0")
+    names = nat.kernel_table()
+    f64 = lambda t: t.float().numpy().astype(np.float64)
+
+    def backward(x, c, dy, tuning, label):
+        y = nat.fwd(x.to(dev), c.to(dev), reverse)
+        dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y.cpu()), reverse)
+        dx, dc = nat.bwd(dy.to(dev), c.to(dev), y, reverse, tuning, out=(_nan_like(y), _nan_like(y)))
+        torch.cuda.synchronize()
+        _check(dx, dx_t, dtype, label + " d_inputs")
+        _check(dc, dc_t, dtype, label + " d_coeffs")
+
+    for shape, teams in [((3, 16384 * 2 + 8), (0, 2, 3)), ((5, 16384 * 3 + 8192), (0, 3)), ((7, 16384 * 5 - 8), (0, 4)),
+                         ((33, 16384 * 4 + 1000), (0, 5)), ((2, 16384 * 13 + 16376), (0, 9)), ((1, 16384 * 40 + 24), (0, 7))]:
+        x, c, dy = _inputs(shape, dtype, shape[0] + shape[1], coeffs="near1")
+        for team in teams:
+            tf = nat.Tuning(D, 16, 2, -1, team)
+            kb = -(-shape[1] // 8192)
+            team_b = min(2 * team, kb)
+            if team_b and shape[1] % 8192 == 0 and kb % team_b:
+                team_b = kb  # (rows of whole such tiles take the kernel for them, whose teams divide the tiles of a row)
+            tb = nat.Tuning(D, 8, 2, -1, team_b) if shape[1] % 8192 else nat.Tuning(D, 16, 1, -1, team_b)
+            pf, pb = nat.plan(x.to(dev), reverse, False, tf), nat.plan(x.to(dev), reverse, True, tb)
+            assert "drift_ragged_w16_s2" in names[pf["kernel_id"]] and pf["tiles_per_row"] == -(-shape[1] // 16384), pf
+            assert ("drift_ragged_w8_s2" in names[pb["kernel_id"]]) == (shape[1] % 8192 != 0) and pb["tiles_per_row"] == kb, pb
+            label = f"{dtype} {shape} rev={reverse} forward team {pf['tasks']}, backward team {pb['tasks']}"
+            _run(nat, x, c, dy, reverse, tf, label, backward_too=False)
+            backward(x, c, dy, tb, label)
+            assert nat.gave_up_count() == 0
+    # the planner's own choice
+    for shape in [(335, 100000), (16, 1000000), (100, 250000)]:
+        x, c, dy = _inputs(shape, dtype, shape[0], coeffs="near1")
+        for is_bwd, geometry in ((False, (16, 2)), (True, (8, 2))):
+            plan = nat.plan(x.to(dev), reverse, is_bwd)
+            assert plan["family"] == D and "ragged" in names[plan["kernel_id"]] and (plan["waves"], plan["slots"]) == geometry, plan
+            assert plan["grid"] <= 256 and plan["grid"] % plan["tasks"] == 0, plan
+        _run(nat, x, c, dy, reverse, None, f"{dtype} {shape} rev={reverse}, default plan")
+    # a poll limit of one: waits run out, the value entering a tile comes from the row's own data instead
+    x, c, dy = _inputs((6, 16384 * 50 + 5000), dtype, 4, coeffs="near1")
+    y_kept = nat.fwd(x.to(dev), c.to(dev), reverse)
+    old = nat.lib().linrec_set_spin_limit(1)
+    try:
+        y = nat.fwd(x.to(dev), c.to(dev), reverse, nat.Tuning(D, 16, 2, -1, 17))
+        dx, dc = nat.bwd(dy.to(dev), c.to(dev), y_kept, reverse, nat.Tuning(D, 8, 2, -1, 33))
+        torch.cuda.synchronize()
+    finally:
+        nat.lib().linrec_set_spin_limit(old)
+    print("16-bit drift with partial tiles, poll limit 1: waits that ran out:", nat.gave_up_count(), flush=True)
     for ws in list(nat._workspaces.values()):
         ws[:16].view(torch.int32)[1] = 0  # (the other tests take a count of zero as the sign that nobody had to fall back)
     _check(y, oracle.fwd(f64(x), f64(c), reverse), dtype, "poll limit 1 outputs")

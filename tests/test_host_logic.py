@@ -343,7 +343,8 @@ class TestPlanner:
         assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
         assert fam((T["team_min_rows"], (1 << 20) + 6)) == nat.FAMILY_TEAM          # few rows that are not whole slots: one team per row
         assert fam((T["team_min_rows"] - 1, (1 << 20) + 6)) == nat.FAMILY_TILE      # fewer: look-back tiles
-        assert fam((300, 65536 + 8), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
+        assert fam((300, 65536 + 4), dtype=torch.bfloat16) == nat.FAMILY_STREAM and fam((96, 65536), dtype=torch.bfloat16) == nat.FAMILY_SWEEP
+        assert fam((300, 65536 + 8), dtype=torch.bfloat16) == D and fam((300, 65536 + 8), True, dtype=torch.bfloat16) == D
         # 16-bit storage: teams whose tiles are stored two steps late serve the backward of up to drift_bwd_max_rows
         # rows of whole tiles of 8192 elements (16 waves of one slot) and the forward of any number of rows of four and
         # more tiles of 16384 elements (16 waves of two slots), where the launch has two (forward: four) tiles for every
@@ -367,7 +368,9 @@ class TestPlanner:
             # rows of 32 tiles and more
             few = T["half_drift_fwd_small_tiles_max_rows"]
             assert fam((few, 8192 * 41), dtype=dt) == D and fam((few + 1, 8192 * 31), dtype=dt) != D
-            assert [fam((n, 8192 * 9), dtype=dt) for n in (128, 300)] == [W, ST]
+            # (rows of an odd number of such tiles: teams with the forward's tiles of 16384 elements, the last one half full,
+            # where they divide the rows evenly; bf16 300 x 73728 27.6 us against 30.3 us for one workgroup per row)
+            assert [fam((n, 8192 * 9), dtype=dt) for n in (128, 200, 300)] == [W, ST, D]
             assert [fam((n, 8192 * 33), dtype=dt) for n in (64, 128, 160, 250, 256)] == [D, D, D, D, ST]
             # a few rows: the tiles per compute unit the table asks for (forward: of 16384 elements)
             for bwd, per_cu, tile in ((False, T["half_drift_fwd_min_tiles_per_cu"], 16384), (True, T["half_drift_bwd_min_tiles_per_cu"], 8192)):
@@ -377,10 +380,12 @@ class TestPlanner:
             assert (q["waves"], q["slots"], q["tasks"], q["grid"]) == (16, 2, 4, 256), q
             assert fam((24, 262144), dtype=dt) == nat.FAMILY_TEAM
             assert fam((24, 262144), True, dtype=dt) == (D if 24 * 32 >= 256 * T["half_drift_bwd_min_tiles_per_cu"] else nat.FAMILY_TEAM)
-            # one or two rows of whole tiles of 4096 elements only: the forward in 8 waves, the backward in look-back tiles
+            # one or two rows of whole tiles of 4096 elements only: the forward in 8 waves, the backward in tiles of 8192
+            # elements, the last one half full
             q = nat.plan(torch.empty(2, 4096 * 1001, dtype=dt))
             assert (q["family"], q["waves"], q["slots"], q["tiles_per_row"]) == (D, 8, 1, 1001), q
-            assert fam((2, 4096 * 1001), True, dtype=dt) == nat.FAMILY_TILE
+            q = nat.plan(torch.empty(2, 4096 * 1001, dtype=dt), False, True)
+            assert (q["family"], q["waves"], q["slots"], q["tiles_per_row"]) == (D, 8, 2, 501), q
             # a caller who names the family and nothing else gets the tiles of 8192 elements where the rows are whole ones
             q = nat.plan(torch.empty(512, 65536, dtype=dt), tuning=nat.Tuning(D))
             assert (q["waves"], q["slots"], q["tasks"]) == (16, 1, 8), q
@@ -388,7 +393,7 @@ class TestPlanner:
             assert [fam((n, 16384), b, dtype=dt) for n in (2048, 4096) for b in (False, True)] == [ST] * 4
             assert fam((1024, 16384), dtype=dt) == nat.FAMILY_TILE and fam((2048, 16000), dtype=dt) == nat.FAMILY_TILE
             # rows beyond one per CU get a launch of their own in the backward only
-            tails = lambda n: [nat.plan(torch.empty(n, 65536 + 8, dtype=dt), False, b)["tail_rows"] for b in (False, True)]
+            tails = lambda n: [nat.plan(torch.empty(n, 65536 + 4, dtype=dt), False, b)["tail_rows"] for b in (False, True)]
             assert tails(288) == [0, 32] and tails(352) == [0, 96] and tails(400) == [0, 0]
         # 16-bit backward with less than two tiles for every compute unit: the teams that wait (from 32 rows on)
         assert fam((100, 32768), True, dtype=torch.bfloat16) == W and fam((100, 32768), dtype=torch.bfloat16) == W
@@ -874,8 +879,14 @@ def test_sixteen_bit_types_plan_and_host_path(dtype):
     assert p["family"] == nat.FAMILY_TILE and p["waves"] * p["slots"] * 64 * 8 >= 4096 and p["slots"] <= 2
     p = nat.plan(torch.empty(16, 1 << 20, dtype=dtype))
     assert p["family"] == nat.FAMILY_DRIFT and p["vec"] == 8
-    p = nat.plan(torch.empty(16, (1 << 20) + 8, dtype=dtype))
+    p = nat.plan(torch.empty(16, (1 << 20) + 4, dtype=dtype))    # rows that are not whole slots
     assert p["family"] == nat.FAMILY_TEAM
+    # rows of whole slots whose last tile is a partial one: drift teams, the backward in 8 waves of two slots
+    pfx = "f16_" if dtype == torch.float16 else "bf16_"
+    p = nat.plan(torch.empty(16, (1 << 20) + 8, dtype=dtype))
+    assert (p["family"], p["waves"], p["slots"], p["tiles_per_row"]) == (nat.FAMILY_DRIFT, 16, 2, 65) and names[p["kernel_id"]] == pfx + "drift_ragged_w16_s2_MODE_FWD_0"
+    p = nat.plan(torch.empty(16, (1 << 20) + 8, dtype=dtype), False, True)
+    assert (p["family"], p["waves"], p["slots"], p["tiles_per_row"]) == (nat.FAMILY_DRIFT, 8, 2, 129) and names[p["kernel_id"]] == pfx + "drift_ragged_w8_s2_MODE_BWD_1"
     p = nat.plan(torch.empty(256, 262144, dtype=dtype).t())
     assert p["family"] == nat.FAMILY_COLUMN and p["vec"] == 4
     p = nat.plan(torch.empty(9, 100, dtype=dtype)[:, 1:])  # base one element past a slot boundary
