@@ -74,9 +74,9 @@ extern "C" {
                                   64 only), fp32 backward 8 x 2 and 16 x 1; 16-bit storage (slots of eight
                                   elements) forward 16 x 2, 16 x 1 and 8 x 1, backward 16 x 1.
                                   The planner's picks are the 16-wave ones, and 8 x 4 forward for fp32 teams beyond 64.
-                                  Rows must be whole tiles; fp32 rows of whole 16-byte slots may end in a partial
-                                  tile (forward 16 x 2 and 8 x 4, backward 16 x 1), and their teams need not divide
-                                  the tiles of a row */
+                                  Rows must be whole tiles; rows of whole 16-byte slots may end in a partial tile
+                                  (fp32 forward 16 x 2 and 8 x 4, backward 16 x 1; 16-bit storage forward 16 x 2,
+                                  backward 8 x 2), and their teams need not divide the tiles of a row */
 
 #define LINREC_FAMILY_COLDRIFT 11 /* as COLUMN in its block form for a few hundred to a few thousand rows: teams
                                    of workgroups share a block of rows and take its steps along the scan axis in
