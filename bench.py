@@ -35,26 +35,26 @@ MEASURED_TRAFFIC_BYTES = {
     ("C1", "tile_w8_s2_v4_MODE_FWD_0_0"): 3.195e6,
     ("C1", "tile_w8_s2_v4_MODE_BWD_1_0"): 5.362e6,
     ("C2", "drift_w8_s4_MODE_FWD_0"): 403.83e6,
-    ("C2", "drift_w16_s2_MODE_FWD_0"): 403.63e6,
+    ("C2", "drift_w16_s2_MODE_FWD_0"): 403.61e6,
     ("C2", "drift_w8_s2_MODE_BWD_1"): 674.74e6,
-    ("C2", "drift_w16_s1_MODE_BWD_1"): 675.47e6,
+    ("C2", "drift_w16_s1_MODE_BWD_1"): 675.45e6,
     ("C2", "stream_w8_s4_MODE_FWD_0"): 402.71e6,
     ("C2", "stream_w8_s4_MODE_BWD_1"): 671.42e6,
     ("C2", "sweep_w8_s4_MODE_BWD_1"): 673.19e6,
     ("C3", "tile_w4_s2_v4_MODE_FWD_1_0"): 402.58e6,
     ("C3", "tile_w4_s2_v4_MODE_BWD_0_0"): 676.67e6,
-    ("C4", "drift_w8_s4_MODE_FWD_0"): 202.36e6,
+    ("C4", "drift_w8_s4_MODE_FWD_0"): 202.30e6,
     ("C4", "sweep_w8_s4_MODE_FWD_0"): 202.13e6,
     ("C4", "sweep_w8_s8_MODE_BWD_1"): 336.69e6,
-    ("C4", "drift_w16_s1_MODE_BWD_1"): 338.47e6,
+    ("C4", "drift_w16_s1_MODE_BWD_1"): 338.40e6,
     ("C5", "column_v2_u8_MODE_FWD_0"): 805.12e6,
     ("C5", "column_v2_u8_MODE_BWD_1"): 1340.78e6,
     ("C2", "bf16_stream_w8_s2_MODE_FWD_0"): 201.40e6,
     ("C2", "bf16_stream_w8_s2_MODE_BWD_1"): 335.63e6,
-    ("C2", "bf16_drift_w16_s2_MODE_FWD_0"): 202.18e6,
-    ("C2", "bf16_drift_w16_s1_MODE_BWD_1"): 337.19e6,
-    ("C4", "bf16_drift_w16_s2_MODE_FWD_0"): 101.30e6,
-    ("C4", "bf16_drift_w16_s1_MODE_BWD_1"): 169.02e6,
+    ("C2", "bf16_drift_w16_s2_MODE_FWD_0"): 202.14e6,
+    ("C2", "bf16_drift_w16_s1_MODE_BWD_1"): 337.22e6,
+    ("C4", "bf16_drift_w16_s2_MODE_FWD_0"): 101.29e6,
+    ("C4", "bf16_drift_w16_s1_MODE_BWD_1"): 169.01e6,
     # the three launches of a segmented scan together (reduce + carry + apply): the inputs are read twice
     ("T1", "segment_apply_v2_u8_MODE_FWD_0"): 1352.9e6,
     ("T1", "colblock_v1_u8_g2_MODE_FWD_0"): 805.16e6,
