@@ -42,7 +42,7 @@ CHAIN_GEOMETRIES = [(4, 2), (4, 4), (8, 2), (8, 4)]
 STREAM_GEOMETRIES = [(4, 4), (8, 2), (8, 4), (16, 2), (8, 8)]
 TEAM_GEOMETRIES = [(4, 2), (4, 4), (8, 2), (8, 4)]
 SWEEP_GEOMETRIES = [(4, 4), (8, 2), (8, 4), (8, 8)]
-DRIFT_GEOMETRIES = [(8, 4), (8, 2), (4, 4), (16, 2), (16, 1), (8, 1)]  # the fp32 backward is compiled for tiles of 4096 elements (8 x 2, 16 x 1); 16-bit storage: 16 x 1 in both passes, 8 x 1 forward
+DRIFT_GEOMETRIES = [(8, 4), (8, 2), (4, 4), (16, 2), (16, 1), (8, 1)]  # the fp32 backward is compiled for tiles of 4096 elements (8 x 2, 16 x 1); 16-bit storage: 16 x 1 in both passes, 16 x 2 and 8 x 1 forward; rows that end in a partial tile: fp32 16 x 2 and 8 x 4 forward, 16 x 1 backward, 16-bit 16 x 2 forward, 8 x 2 backward
 
 
 def candidates(t):
