@@ -113,6 +113,63 @@ def test_random_layout(seed):
         assert rep["normwise"] <= tol, (what, case, rep)
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_random_long_and_short_rows_through_the_default_plan(seed):
+    """Dense row-major tensors at the sizes where the planner's long-row kernels take over (up to 4e7 elements), 40
+    seeded cases each: rows of whole tiles, rows of whole slots that end in a partial tile (few and many of them), one to
+    five very long rows, arbitrary lengths, and short rows down to two elements.  Both passes through the C ABI with the
+    default plan, result buffers poisoned, against the float64 recurrence; 16-bit results to half a unit in the last
+    place."""
+    from linrec_amd import _native as nat
+    rng = np.random.default_rng(7000 + seed)
+    dev = torch.device("cuda:0")
+    names = nat.kernel_table()
+    f64 = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    for case in range(40):
+        dtype = DTYPES[int(rng.integers(3))]
+        fv = 4 if dtype == torch.float32 else 8
+        kind = int(rng.integers(6))
+        if kind == 0:    # short dense rows
+            L, n = int(rng.integers(2, 70)), int(rng.integers(2, 5000))
+        elif kind == 1:  # whole slots, a partial last tile
+            tile = 8192 if dtype == torch.float32 else 16384
+            L = int(rng.integers(2, 40)) * (tile // 2) + int(rng.integers(1, tile // fv)) * fv
+            n = int(rng.choice([1, 2, 3, 5, 16, 33, 100, 257, 300, 600]))
+        elif kind == 2:  # whole tiles
+            L, n = int(rng.integers(1, 30)) * 8192, int(rng.choice([1, 2, 4, 16, 64, 130, 256, 300, 512]))
+        elif kind == 3:  # arbitrary lengths
+            L, n = int(rng.integers(100, 200000)), int(rng.integers(1, 400))
+        elif kind == 4:  # a few thousand elements
+            L, n = int(rng.integers(200, 9000)), int(rng.integers(1, 3000))
+        else:            # a few very long rows
+            L, n = int(rng.integers(200000, 3000000)), int(rng.integers(1, 6))
+        if n * L > 40_000_000:
+            n = max(1, 40_000_000 // L)
+        reverse = bool(rng.integers(2))
+        g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+        x = torch.randn(n, L, generator=g).to(dtype)
+        c = (torch.rand(n, L, generator=g) * (0.2 if L > 4000 else 1.8) + (0.8 if L > 4000 else -0.9)).to(dtype)
+        dy = torch.randn(n, L, generator=g).to(dtype)
+        xd, cd, dyd = x.to(dev), c.to(dev), dy.to(dev)
+        kernels = [names[nat.plan(xd, reverse, b)["kernel_id"]] for b in (False, True)]
+        what = (seed, case, str(dtype), (n, L), reverse, kernels)
+        print(*what, flush=True)
+        y = nat.fwd(xd, cd, reverse, None, out=torch.full_like(xd, float("nan")))
+        dx, dc = nat.bwd(dyd, cd, y, reverse, None, out=(torch.full_like(xd, float("nan")), torch.full_like(xd, float("nan"))))
+        torch.cuda.synchronize()
+        y_t = oracle.fwd(f64(x), f64(c), reverse)
+        dx_t, dc_t = oracle.bwd(f64(dy), f64(c), f64(y), reverse)  # from the outputs the forward stored
+        for got, want, name in ((y, y_t, "outputs"), (dx, dx_t, "d_inputs"), (dc, dc_t, "d_coeffs")):
+            got = f64(got)
+            assert np.isfinite(got).all(), (name, what)
+            if dtype == torch.float32:
+                assert np.abs(got - want).max() <= 2e-5 * max(np.abs(want).max(), 1e-30), (name, what)
+            else:
+                unit = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 1e-30))) - (10 if dtype == torch.float16 else 7))
+                assert (np.abs(got - want) <= 0.51 * unit + 1e-5 * np.abs(want).max()).all(), (name, what)
+    assert nat.gave_up_count() == 0
+
+
 def _view_of(t, ops):
     """`t` after a sequence of view-making operations (op, dim, argument); operations that do not apply
     to the tensor at hand are skipped."""
