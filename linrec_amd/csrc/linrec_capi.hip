@@ -686,7 +686,20 @@ int make_plan(const Problem& q, const linrec_tuning_t* tune, linrec_plan_t* out)
       if (q.base_mis >= 0 && full_slots > kLongRowSlots) {
         if (drift_slots_for(q, fv) > 0) family = LINREC_FAMILY_DRIFT;
         else if (sweep_slots_for(q, fv) > 0) family = LINREC_FAMILY_SWEEP;
-        else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) family = LINREC_FAMILY_STREAM;
+        else if (q.numseq >= q.at(kStreamMinRows - 1) + 1) {
+          family = LINREC_FAMILY_STREAM;
+          // fp32 rows from a length on (generated table): look-back tiles of 16384 elements, which the dispatcher hands
+          // to whichever compute unit is free (rows that are not whole slots, forward / backward in us against one
+          // workgroup per row: 335 x 100001 74.7 / 134.7 against 91.7 / 159.0, 300 x 65541 47.3 / 81.8 against 58.5 / 98.9,
+          // 4096 x 65541 522 / 975 against 613 / 1067, 8192 x 32770 534 / 1018 against 612 / 1078; but 2000 x 20001
+          // 99.9 / 177.6 against 92.0 / 160.8; 16-bit storage, tiles of eight waves of four slots: 512 x 65542 58.7 / 86.8
+          // against 42.0 / 73.0)
+          // (rows of whole slots stay where the rules above left them; a caller that can only give so much workspace is
+          // served by the kernel that needs none)
+          if (!half && q.seqlen >= kT_stream_max_len && !(rows_on_slots && q.seqlen % fv == 0) &&
+              !(q.workspace_cap && linrec_workspace_bytes_for_tiles(q.numseq * ceil_div(full_slots, int64_t(8) * 8 * 64)) > q.workspace_cap))
+            family = LINREC_FAMILY_TILE;
+        }
         else if (q.numseq >= (half ? (q.is_bwd ? kTeamMinRowsHalfBwd : kTeamMinRowsHalfFwd) : kTeamMinRows)) family = LINREC_FAMILY_TEAM;
       }
       // 16-bit storage, many rows of exactly two of the stream kernel's tiles (16384 elements): one workgroup of

@@ -300,6 +300,9 @@ CROSSOVERS = [
     Crossover("stream_min_rows", "long rows that are not whole slots (65542 elements): one team of workgroups per row "
               "against one workgroup per row, by the number of rows", [64, 96, 112, 128, 129, 144, 160, 192],
               lambda v: (v, 65542), _both(_t(nat.FAMILY_TEAM)), _both(_t(nat.FAMILY_STREAM))),
+    Crossover("stream_max_len", "600 long rows that are not whole slots: one workgroup per row against look-back tiles of "
+              "16384 elements, by the row length", [16386, 20002, 24578, 28002, 32770, 40002, 49154, 65542],
+              lambda v: (600, v), _both(_t(nat.FAMILY_STREAM)), _both(_t(nat.FAMILY_TILE, 8, 8, 1, 1))),
     Crossover("team_min_rows", "a few very long rows that are not whole slots (1048582 elements): look-back tiles against "
               "one team of 64 workgroups per row, by the number of rows", [2, 3, 4, 5, 6, 8, 12],
               lambda v: (v, 1048582), _both(_t(nat.FAMILY_TILE, 8, 8, 1, 1)), _both(_t(nat.FAMILY_TEAM))),

@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 
 CASES = {
     # name: (numseq, seqlen, transposed, reverse, dtype, expected family)
-    "stream_f32": (70144, 32778, False, False, torch.float32, "STREAM"),       # rows that are not whole slots
+    "stream_f32": (90000, 24578, False, False, torch.float32, "STREAM"),       # rows that are not whole slots
+    "lookback_f32": (70144, 32778, False, False, torch.float32, "TILE"),       # ... and long enough for look-back tiles
     "drift_ragged_f32": (70144, 32776, False, False, torch.float32, "DRIFT"),  # whole slots, a partial last tile
     "drift_rows_f32": (56000, 40960, False, False, torch.float32, "DRIFT"),  # (its backward: teams that wait, SWEEP)
     "tile_f32": (1100000, 2048, False, True, torch.float32, "TILE"),

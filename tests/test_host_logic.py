@@ -110,8 +110,8 @@ def test_planner_follows_the_compute_unit_count():
                 if c["family"] == nat.FAMILY_COLDRIFT:
                     assert c["grid"] == 64 * c["tasks"] <= cus
             # one workgroup per row from half the CUs on, teams below
-            assert nat.plan(torch.empty(cus // 2 + 1, 65542))["family"] == nat.FAMILY_STREAM
-            assert nat.plan(torch.empty(cus // 2, 65542))["family"] == nat.FAMILY_TEAM
+            assert nat.plan(torch.empty(cus // 2 + 1, 24578))["family"] == nat.FAMILY_STREAM
+            assert nat.plan(torch.empty(cus // 2, 24578))["family"] == nat.FAMILY_TEAM
         assert seen[(256, False)] == 256 and seen[(128, False)] == 128 and seen[(64, False)] == 64
         assert seen[(256, True)] == 256 and seen[(128, True)] == 128 and seen[(64, True)] == 64
         # a team that cannot be resident at once is refused rather than left to wait for absent mates
@@ -324,7 +324,12 @@ class TestPlanner:
         assert (q["family"], q["waves"], q["slots"], q["tasks"], q["grid"]) == (D, 16, 2, 8, 256), q
         m = T["drift_bwd_max_rows"]
         assert 1024 <= m and fam((m, 65536), True) == D and fam((m + 256, 65536), True) == W
-        assert fam((m + 256, 131072), True) == ST and fam((4096, 65536 + 6)) == ST and fam((4096, 65536 + 8)) == D
+        assert fam((m + 256, 131072), True) == ST and fam((4096, 24576 + 6)) == ST and fam((4096, 65536 + 8)) == D
+        # rows that are not whole slots, from the generated length on: look-back tiles of 16384 elements
+        assert fam((4096, T["stream_max_len"] - 4)) == ST and fam((4096, T["stream_max_len"])) == nat.FAMILY_TILE and T["stream_max_len"] % 4
+        q = nat.plan(torch.empty(300, 65536 + 6))
+        assert (q["family"], q["waves"], q["slots"], q["carry"], q["tiles_per_row"]) == (nat.FAMILY_TILE, 8, 8, 1, 5), q
+        assert fam((300, 65536 + 6), dtype=torch.bfloat16) == ST   # (16-bit storage: one workgroup per row)
         assert fam((3, 1 << 20)) == nat.FAMILY_TILE   # three tiles for every workgroup of a team of the whole chip: too few
         slots = lambda shape, bwd=False: nat.plan(torch.empty(shape), False, bwd)["slots"]
         # stream tiles of 16384 elements: long rows of whole such tiles, or many rows
@@ -332,14 +337,14 @@ class TestPlanner:
         assert slots((256, 32768 + 8192)) == 4
         # tiles of 4096 elements where they pad the row less, and for rows up to 16384 elements
         assert slots((1024, 16384)) == 2 and slots((3355, 10000)) == 2 and slots((1677, 20000)) == 2
-        assert slots((700, 24576)) == 4 and slots((838, 40002)) == 4 and slots((800, 36002)) == 2
-        assert fam((300, 65536 + 6)) == nat.FAMILY_STREAM          # rows that are not whole slots
+        assert slots((700, 24576)) == 4 and slots((838, 24570)) == 4 and slots((800, 26002)) == 2
+        assert fam((300, 24576 + 6)) == nat.FAMILY_STREAM          # rows that are not whole slots
         assert fam((300, 65536 + 4)) == D and fam((838, 40000)) == D   # whole slots, a partial last tile: drift teams
         # ... whose rows beyond one per CU, if few, go to a second launch of their own (teams per row)
-        p = nat.plan(torch.empty(300, 65536 + 6))
+        p = nat.plan(torch.empty(300, 24576 + 6))
         assert (p["tail_rows"], p["grid"]) == (44, 256) and p["workspace_bytes"] > 0
-        assert [nat.plan(torch.empty(n, 65536 + 6))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
-        assert nat.plan(torch.empty(300, 65536 + 6), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
+        assert [nat.plan(torch.empty(n, 24576 + 6))["tail_rows"] for n in (256, 257, 352, 353, 600)] == [0, 1, 96, 0, 0]
+        assert nat.plan(torch.empty(300, 24576 + 6), tuning=nat.Tuning(nat.FAMILY_STREAM))["tail_rows"] == 0
         assert fam((300, 12288)) == nat.FAMILY_STREAM              # three tiles per row: not worth an exchange
         assert fam((T["team_min_rows"], (1 << 20) + 6)) == nat.FAMILY_TEAM          # few rows that are not whole slots: one team per row
         assert fam((T["team_min_rows"] - 1, (1 << 20) + 6)) == nat.FAMILY_TILE      # fewer: look-back tiles
@@ -609,7 +614,7 @@ class TestPlanner:
         assert lib.linrec_plan_f32(None, 4, 10, 5, 1, 0, 0, None, ctypes.byref(plan)) == -1  # rows overlap
         assert lib.linrec_plan_f32(None, 4, 2 ** 31, 2 ** 31, 1, 0, 0, None, ctypes.byref(plan)) == -4
         assert lib.linrec_workspace_bytes(16, 1 << 20, 1 << 20, 1, 0, 0, None) > 0
-        assert lib.linrec_workspace_bytes(4096, 65542, 65542, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
+        assert lib.linrec_workspace_bytes(4096, 24582, 24582, 1, 0, 0, None) == 0  # one workgroup per row: nobody waits
         assert lib.linrec_workspace_bytes_for_tiles(0) == 0
         assert lib.linrec_workspace_bytes_for_tiles(1000) >= 16 + 16 * 1000
 
